@@ -1,0 +1,388 @@
+/*
+ * CPU oracle for the go-metal optimizer step (see oracle.h).  TEST
+ * INFRASTRUCTURE ONLY: nothing in the shipped library links this file.
+ *
+ * Every statement below is one node of the reference's MPSGraph op chain and
+ * performs exactly one binary32 rounding.  Build flags that this relies on:
+ * -ffp-contract=off (no FMA fusion), no -ffast-math, SSE scalar/vector math
+ * (IEEE division and square root), denormals left enabled.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <string.h>
+
+#define GM_PARALLEL_FOR _Pragma("omp parallel for schedule(static) num_threads(nt) if(nt > 1)")
+
+static int clamp_threads(int nthreads) { return nthreads < 1 ? 1 : nthreads; }
+
+/* bridge_optimizer.m:398-399 */
+void gm_oracle_bias_corrections(float beta1, float beta2, int step, float *bc1, float *bc2)
+{
+    *bc1 = 1.0f - powf(beta1, (float)step);
+    *bc2 = 1.0f - powf(beta2, (float)step);
+}
+
+/* bridge_optimizer.m:2066 (momentum_schedule_next; the :2065 value is unused there) */
+float gm_oracle_nadam_mu_next(float beta1, int step)
+{
+    float exponent = (float)(step + 1) * 0.004f;
+    float decay = powf(0.96f, exponent);
+    float half_decay = 0.5f * decay;
+    float one_minus = 1.0f - half_decay;
+    return beta1 * one_minus;
+}
+
+/* bridge_optimizer.m:160-357 */
+void gm_oracle_sgd_step(float *w, const float *g, float *m, size_t n,
+                        float lr, float momentum, float weight_decay, int nesterov,
+                        int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    const int use_momentum = (momentum > 0.0f) && (m != NULL);   /* :233 */
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) {
+        float wi = w[i];
+        float gi = g[i];
+        if (weight_decay > 0.0f) {          /* :219-228 */
+            float decay = wi * weight_decay;
+            gi = gi + decay;
+        }
+        if (use_momentum) {
+            float scaled = m[i] * momentum;  /* :245 */
+            float mi = scaled + gi;          /* :248 */
+            float upd;
+            if (nesterov != 0) {             /* :257-267 */
+                float t1 = momentum * mi;
+                float t2 = t1 + gi;
+                upd = lr * t2;
+            } else {                         /* :270-272 */
+                upd = lr * mi;
+            }
+            w[i] = wi - upd;                 /* :276 */
+            m[i] = mi;
+        } else {                             /* :315-322 */
+            float upd = lr * gi;
+            w[i] = wi - upd;
+        }
+    }
+}
+
+/* One element of bridge_optimizer.m:484-550; shared with the AMP step. */
+static inline void adam_element(float *w, float g, float *m, float *v,
+                                float lr, float beta1, float beta2,
+                                float one_minus_beta1, float one_minus_beta2,
+                                float eps, float weight_decay, float bc1, float bc2)
+{
+    float wi = *w;
+    float m_scaled = *m * beta1;               /* :484 */
+    float g_scaled = g * one_minus_beta1;      /* :487 */
+    float mi = m_scaled + g_scaled;            /* :490 */
+    float g_sq = g * g;                        /* :495 */
+    float v_scaled = *v * beta2;               /* :498 */
+    float g_sq_scaled = g_sq * one_minus_beta2;/* :501 */
+    float vi = v_scaled + g_sq_scaled;         /* :504 */
+    float m_hat = mi / bc1;                    /* :509 */
+    float v_hat = vi / bc2;                    /* :514 */
+    float root = sqrtf(v_hat);                 /* :519 */
+    float den = root + eps;                    /* :521 */
+    float upd = m_hat / den;                   /* :526 */
+    if (weight_decay > 0.0f) {                 /* :531-540 */
+        float decay = wi * weight_decay;
+        upd = upd + decay;
+    }
+    float scaled = upd * lr;                   /* :543 */
+    *w = wi - scaled;                          /* :548 */
+    *m = mi;
+    *v = vi;
+}
+
+/* bridge_optimizer.m:360-641 */
+void gm_oracle_adam_step(float *w, const float *g, float *m, float *v, size_t n,
+                         float lr, float beta1, float beta2, float eps, float weight_decay,
+                         int step, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    float bc1, bc2;
+    gm_oracle_bias_corrections(beta1, beta2, step, &bc1, &bc2);
+    const float omb1 = 1.0f - beta1;           /* :469 */
+    const float omb2 = 1.0f - beta2;           /* :471 */
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++)
+        adam_element(&w[i], g[i], &m[i], &v[i], lr, beta1, beta2, omb1, omb2,
+                     eps, weight_decay, bc1, bc2);
+}
+
+/* bridge_optimizer.m:691-951 */
+void gm_oracle_rmsprop_step(float *w, const float *g, float *s, float *mom, float *gavg, size_t n,
+                            float lr, float alpha, float eps, float weight_decay,
+                            float momentum, int centered, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    const float oma = 1.0f - alpha;            /* :773 */
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) {
+        float wi = w[i];
+        float gi = g[i];
+        float g_sq = gi * gi;                  /* :782 */
+        float s_scaled = s[i] * alpha;         /* :785 */
+        float g_sq_scaled = g_sq * oma;        /* :788 */
+        float si = s_scaled + g_sq_scaled;     /* :791 */
+        float den;
+        if (centered) {                        /* :797-824 */
+            float ga_scaled = gavg[i] * alpha;
+            float g_term = gi * oma;
+            float ga = ga_scaled + g_term;
+            float ga_sq = ga * ga;
+            float var = si - ga_sq;
+            float var_eps = var + eps;
+            den = sqrtf(var_eps);
+            gavg[i] = ga;
+        } else {                               /* :827-830 */
+            float s_eps = si + eps;
+            den = sqrtf(s_eps);
+        }
+        float upd = gi / den;                  /* :834 */
+        if (momentum > 0.0f) {                 /* :839-854 */
+            float b_scaled = mom[i] * momentum;
+            float bi = b_scaled + upd;
+            mom[i] = bi;
+            upd = bi;
+        }
+        if (weight_decay > 0.0f) {             /* :857-866 */
+            float decay = wi * weight_decay;
+            upd = upd + decay;
+        }
+        float scaled = upd * lr;               /* :869 */
+        w[i] = wi - scaled;                    /* :874 */
+        s[i] = si;
+    }
+}
+
+/* bridge_optimizer.m:1421-1588 */
+void gm_oracle_adagrad_step(float *w, const float *g, float *s, size_t n,
+                            float lr, float eps, float weight_decay, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) {
+        float wi = w[i];
+        float gi = g[i];
+        if (weight_decay > 0.0f) {             /* :1480-1488 */
+            float decay = wi * weight_decay;
+            gi = gi + decay;
+        }
+        float g_sq = gi * gi;                  /* :1492 */
+        float si = s[i] + g_sq;                /* :1495 */
+        float root = sqrtf(si);                /* :1501 */
+        float den = root + eps;                /* :1503 */
+        float alr = lr / den;                  /* :1506 */
+        float upd = alr * gi;                  /* :1512 */
+        w[i] = wi - upd;                       /* :1515 */
+        s[i] = si;
+    }
+}
+
+/* bridge_optimizer.m:1708-1925 */
+void gm_oracle_adadelta_step(float *w, const float *g, float *s, float *a, size_t n,
+                             float rho, float eps, float weight_decay, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    const float omr = 1.0f - rho;
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) {
+        float wi = w[i];
+        float gi = g[i];
+        float ai = a[i];
+        if (weight_decay > 0.0f) {             /* :1773-1781 */
+            float decay = wi * weight_decay;
+            gi = gi + decay;
+        }
+        float g_sq = gi * gi;                  /* :1785 */
+        float s_scaled = s[i] * rho;           /* :1788 */
+        float g_sq_scaled = g_sq * omr;        /* :1791 */
+        float si = s_scaled + g_sq_scaled;     /* :1794 */
+        float s_eps = si + eps;                /* :1800 */
+        float rms_g = sqrtf(s_eps);            /* :1803 */
+        float a_eps = ai + eps;                /* :1807 */
+        float rms_u = sqrtf(a_eps);            /* :1810 */
+        float alr = rms_u / rms_g;             /* :1815 */
+        float d = alr * gi;                    /* :1818 */
+        float neg_d = -d;                      /* :1821 */
+        w[i] = wi + neg_d;                     /* :1826 */
+        float d_sq = neg_d * neg_d;            /* :1832 */
+        float a_scaled = ai * rho;             /* :1835 */
+        float d_sq_scaled = d_sq * omr;        /* :1838 */
+        a[i] = a_scaled + d_sq_scaled;         /* :1841 */
+        s[i] = si;
+    }
+}
+
+/* bridge_optimizer.m:2023-2280 */
+void gm_oracle_nadam_step(float *w, const float *g, float *m, float *v, size_t n,
+                          float lr, float beta1, float beta2, float eps, float weight_decay,
+                          int step, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    float bc1, bc2;
+    gm_oracle_bias_corrections(beta1, beta2, step, &bc1, &bc2);   /* :2061-2062 */
+    const float mu = gm_oracle_nadam_mu_next(beta1, step);        /* :2066 */
+    const float one_minus_mu = 1.0f - mu;                         /* :2153 */
+    const float omb1 = 1.0f - beta1;
+    const float omb2 = 1.0f - beta2;
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) {
+        float wi = w[i];
+        float gi = g[i];
+        float m_scaled = m[i] * beta1;          /* :2114 */
+        float g_scaled = gi * omb1;             /* :2117 */
+        float mi = m_scaled + g_scaled;         /* :2120 */
+        float g_sq = gi * gi;                   /* :2125 */
+        float v_scaled = v[i] * beta2;          /* :2128 */
+        float g_sq_scaled = g_sq * omb2;        /* :2131 */
+        float vi = v_scaled + g_sq_scaled;      /* :2134 */
+        float v_hat = vi / bc2;                 /* :2139 */
+        float m_hat = mi / bc1;                 /* :2145 */
+        float g_hat = gi / bc1;                 /* :2148 */
+        float m_term = m_hat * mu;              /* :2158 */
+        float g_term = g_hat * one_minus_mu;    /* :2161 */
+        float m_bar = m_term + g_term;          /* :2164 */
+        float root = sqrtf(v_hat);              /* :2170 */
+        float den = root + eps;                 /* :2171 */
+        float upd = m_bar / den;                /* :2176 */
+        if (weight_decay > 0.0f) {              /* :2181-2190 */
+            float decay = wi * weight_decay;
+            upd = upd + decay;
+        }
+        float scaled = upd * lr;                /* :2193 */
+        w[i] = wi - scaled;                     /* :2198 */
+        m[i] = mi;
+        v[i] = vi;
+    }
+}
+
+/* ---- fp16 casts, bridge_memory.m:361-377 ---- */
+
+uint16_t gm_oracle_f32_to_f16(float x)
+{
+    uint32_t u;
+    memcpy(&u, &x, sizeof u);
+    uint32_t sign = (u >> 16) & 0x8000u;
+    uint32_t exp = (u >> 23) & 0xFFu;
+    uint32_t man = u & 0x7FFFFFu;
+    if (exp == 0xFFu) {                         /* inf / NaN */
+        if (man == 0) return (uint16_t)(sign | 0x7C00u);
+        /* quiet NaN, keep the top payload bits */
+        return (uint16_t)(sign | 0x7E00u | (man >> 13));
+    }
+    int32_t e = (int32_t)exp - 127 + 15;        /* biased half exponent */
+    if (e >= 0x1F) return (uint16_t)(sign | 0x7C00u);   /* overflow before rounding */
+    if (e <= 0) {
+        /* subnormal half or zero: value = 1.man * 2^(exp-127), ulp = 2^-24 */
+        if (e < -10) return (uint16_t)sign;     /* below half of the smallest subnormal */
+        uint32_t full = man | 0x800000u;        /* 24-bit significand */
+        uint32_t shift = (uint32_t)(14 - e);    /* 14..24 */
+        uint32_t q = full >> shift;
+        uint32_t rem = full & ((1u << shift) - 1u);
+        uint32_t halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (q & 1u))) q++;
+        return (uint16_t)(sign | q);            /* q may carry into the normal range */
+    }
+    uint32_t q = ((uint32_t)e << 10) | (man >> 13);
+    uint32_t rem = man & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++;   /* may carry up to inf */
+    return (uint16_t)(sign | q);
+}
+
+float gm_oracle_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t u;
+    if (exp == 0x1Fu) {
+        u = sign | 0x7F800000u | (man << 13);
+    } else if (exp != 0) {
+        u = sign | ((exp - 15 + 127) << 23) | (man << 13);
+    } else if (man == 0) {
+        u = sign;
+    } else {
+        /* subnormal half: normalise */
+        int e = -1;
+        do { e++; man <<= 1; } while ((man & 0x400u) == 0);
+        u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+    }
+    float f;
+    memcpy(&f, &u, sizeof f);
+    return f;
+}
+
+void gm_oracle_convert_f32_to_f16(const float *src, uint16_t *dst, size_t n, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) dst[i] = gm_oracle_f32_to_f16(src[i]);
+}
+
+void gm_oracle_convert_f16_to_f32(const uint16_t *src, float *dst, size_t n, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < n; i++) dst[i] = gm_oracle_f16_to_f32(src[i]);
+}
+
+/* ---- mixed-precision Adam ---- */
+
+int gm_oracle_amp_found_inf(const uint16_t *const *g16, const size_t *n, int num_tensors, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    int found = 0;
+    for (int t = 0; t < num_tensors; t++) {
+        const uint16_t *g = g16[t];
+        const size_t cnt = n[t];
+        int local = 0;
+        #pragma omp parallel for schedule(static) num_threads(nt) if(nt > 1) reduction(|:local)
+        for (size_t i = 0; i < cnt; i++)
+            local |= ((g[i] & 0x7C00u) == 0x7C00u);
+        found |= local;
+    }
+    return found;
+}
+
+int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *const *m,
+                            float *const *v, uint16_t *const *w16, const size_t *n, int num_tensors,
+                            float lr, float beta1, float beta2, float eps, float weight_decay,
+                            gm_oracle_amp_state *st, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    if (gm_oracle_amp_found_inf(g16, n, num_tensors, nthreads)) {
+        st->scale = st->scale * st->backoff_factor;
+        st->growth_tracker = 0;
+        return 1;
+    }
+    st->step_count += 1;
+    float bc1, bc2;
+    gm_oracle_bias_corrections(beta1, beta2, (int)st->step_count, &bc1, &bc2);
+    const float omb1 = 1.0f - beta1;
+    const float omb2 = 1.0f - beta2;
+    const float inv_scale = 1.0f / st->scale;
+    for (int t = 0; t < num_tensors; t++) {
+        float *wt = w[t], *mt = m[t], *vt = v[t];
+        const uint16_t *gt = g16[t];
+        uint16_t *ht = w16[t];
+        const size_t cnt = n[t];
+        GM_PARALLEL_FOR
+        for (size_t i = 0; i < cnt; i++) {
+            float gi = gm_oracle_f16_to_f32(gt[i]) * inv_scale;
+            adam_element(&wt[i], gi, &mt[i], &vt[i], lr, beta1, beta2, omb1, omb2,
+                         eps, weight_decay, bc1, bc2);
+            ht[i] = gm_oracle_f32_to_f16(wt[i]);
+        }
+    }
+    st->growth_tracker += 1;
+    if (st->growth_tracker == st->growth_interval) {
+        st->scale = st->scale * st->growth_factor;
+        st->growth_tracker = 0;
+    }
+    return 0;
+}
