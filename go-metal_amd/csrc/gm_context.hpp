@@ -1,0 +1,60 @@
+// Process-wide state behind the C ABI: the device context (one HIP stream per
+// GPU), the registry that remembers the byte length of every buffer handed out
+// by allocate_metal_buffer, and the per-thread error message.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace gm {
+
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+
+// true when the HIP call succeeded; otherwise records "what: <hip error>".
+bool hip_ok(hipError_t e, const char *what);
+
+struct MultiTensorPlan;
+
+struct Context {
+    int device_id = 0;
+    bool usable = false;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    std::atomic<int> refs{0};
+    std::mutex mu;                                    // guards plans and launches
+    std::vector<std::unique_ptr<MultiTensorPlan>> plans;  // most recently used first
+    ~Context();
+};
+
+// The context of HIP device 0, created on first call; nullptr if no GPU works.
+Context *default_context();
+
+// Maps a device handle from the C ABI to a context.  Any non-zero handle
+// resolves to the default context: as on Metal, every device handle aliases
+// the one system GPU, and tests may pass placeholder handles.
+Context *resolve_device(uintptr_t device);
+
+// Makes ctx's GPU current on the calling thread (HIP's current device is
+// thread-local and callers may hop threads between calls).
+bool make_current(Context *ctx);
+
+// ---- buffer registry: handle (device address) -> allocation length ----
+void registry_add(uintptr_t buffer, size_t bytes);
+void registry_remove(uintptr_t buffer);
+// 0 when the handle is not one of ours.
+size_t registry_length(uintptr_t buffer);
+// Bumped on every removal; cached launch plans are only valid for the
+// generation they were built in (a freed address may come back with a
+// different length).
+uint64_t registry_generation();
+
+}  // namespace gm

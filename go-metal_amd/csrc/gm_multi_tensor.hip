@@ -1,0 +1,885 @@
+// Multi-tensor-apply optimizer steps for gfx950: plan cache, update kernels and
+// the execute_*_step entry points of the C ABI (the HIP counterpart of
+// cgo_bridge/bridge_optimizer.m).
+//
+// One launch per step.  Workgroup b walks chunk b of the device-side chunk
+// table: 256 lanes, each lane moving 16-byte vectors (global_load_dwordx4 /
+// global_store_dwordx4), UNROLL vectors of every stream in flight before the
+// first use, every state read once and written once, fp32 throughout.  The
+// path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS staging and
+// no MFMA, only enough independent loads per lane to cover HBM latency.
+#include "gm_context.hpp"
+#include "gm_plan.hpp"
+#include "gm_rules.hpp"
+
+#include "../../include/gometal_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+namespace gm {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+constexpr int kChunkGranule = kBlock * 4 * kUnroll;   // elements one pass of a workgroup covers
+constexpr int kDefaultChunkElements = kChunkGranule;
+constexpr size_t kMaxCachedPlans = 16;
+
+static std::atomic<int> g_chunk_elements{kDefaultChunkElements};
+static std::atomic<int> g_nontemporal{1};
+
+int current_chunk_elements() { return g_chunk_elements.load(); }
+bool current_nontemporal() { return g_nontemporal.load() != 0; }
+
+// ------------------------------------------------------------------ plan ----
+MultiTensorPlan::~MultiTensorPlan()
+{
+    if (d_recs) (void)hipFree(d_recs);
+    if (d_chunks) (void)hipFree(d_chunks);
+}
+
+static bool plan_matches(const MultiTensorPlan &p, const PlanRequest &r, int chunk, uint64_t gen)
+{
+    if (p.kind != r.kind || p.variant != r.variant || p.num_tensors != r.num_tensors ||
+        p.chunk_elements != chunk || p.generation != gen)
+        return false;
+    const size_t n = (size_t)r.num_tensors;
+    if (n == 0) return true;
+    if (std::memcmp(p.sizes.data(), r.sizes, n * sizeof(int)) != 0) return false;
+    for (int k = 0; k < kNumSlots; k++) {
+        const uintptr_t *cached = p.handles.data() + (size_t)k * n;
+        if (r.slot[k]) {
+            if (std::memcmp(cached, r.slot[k], n * sizeof(uintptr_t)) != 0) return false;
+        } else {
+            for (size_t i = 0; i < n; i++)
+                if (cached[i] != 0) return false;
+        }
+    }
+    return true;
+}
+
+static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanRequest &r, int chunk,
+                                                   uint64_t gen)
+{
+    auto plan = std::make_unique<MultiTensorPlan>();
+    const size_t n = (size_t)r.num_tensors;
+    plan->kind = r.kind;
+    plan->variant = r.variant;
+    plan->num_tensors = r.num_tensors;
+    plan->chunk_elements = chunk;
+    plan->generation = gen;
+    plan->sizes.assign(r.sizes, r.sizes + n);
+    plan->handles.assign((size_t)kNumSlots * n, 0);
+    for (int k = 0; k < kNumSlots; k++)
+        if (r.slot[k]) std::memcpy(plan->handles.data() + (size_t)k * n, r.slot[k], n * sizeof(uintptr_t));
+
+    std::vector<TensorRec> recs;
+    std::vector<Chunk> chunks;
+    recs.reserve(n);
+    for (size_t i = 0; i < n; i++) {
+        uintptr_t h[kNumSlots];
+        for (int k = 0; k < kNumSlots; k++) h[k] = plan->handles[(size_t)k * n + i];
+
+        // 1. handles that must be present
+        bool skip = false;
+        for (int k = 0; k < kNumSlots && plan->status == 0; k++) {
+            if (h[k] != 0) continue;
+            if (r.required_mask & (1u << k)) {
+                if (r.missing_code != 0) plan->status = r.missing_code;
+                else skip = true;
+            } else if (r.skip_if_zero_mask & (1u << k)) {
+                skip = true;
+            }
+        }
+        if (plan->status == 0 && r.extra_check) plan->status = r.extra_check(r, (int)i);
+        if (plan->status != 0) break;
+
+        const int size_bytes = r.sizes[i] > 0 ? r.sizes[i] : 0;
+        const size_t numel = (size_t)size_bytes / sizeof(float);
+        if (skip || numel == 0) continue;
+
+        // 2. an allocation of ours that is shorter than the tensor: skip it
+        //    (bridge_optimizer.m:427-436)
+        uint32_t flags = kRecVectorOk | kRecGrad16VectorOk;
+        for (int k = 0; k < kNumSlots; k++) {
+            if (h[k] == 0) continue;
+            const bool half = (r.half_mask & (1u << k)) != 0;
+            const size_t need = numel * (half ? 2 : 4);
+            const size_t have = registry_length(h[k]);
+            if (have != 0 && have < need) skip = true;
+            if (h[k] % (half ? 8 : 16) != 0) flags &= ~kRecVectorOk;
+            if (half && k == kSlotGrad && h[k] % 16 != 0) flags &= ~kRecGrad16VectorOk;
+        }
+        if (skip) continue;
+
+        TensorRec rec;
+        for (int k = 0; k < kNumSlots; k++) rec.p[k] = reinterpret_cast<void *>(h[k]);
+        rec.flags = flags;
+        rec.pad = 0;
+        const uint32_t rec_index = (uint32_t)recs.size();
+        recs.push_back(rec);
+        for (size_t off = 0; off < numel; off += (size_t)chunk) {
+            const size_t left = numel - off;
+            chunks.push_back(Chunk{rec_index, (uint32_t)(left < (size_t)chunk ? left : (size_t)chunk), off});
+        }
+        plan->total_elements += numel;
+    }
+    if (plan->status != 0 || chunks.empty()) return plan;
+    if (chunks.size() > 0x7FFFFFFFull) {
+        set_error("parameter list needs %zu chunks, more than one launch can address", chunks.size());
+        return nullptr;
+    }
+
+    if (!hip_ok(hipMalloc(&plan->d_recs, recs.size() * sizeof(TensorRec)), "hipMalloc(recs)") ||
+        !hip_ok(hipMalloc(&plan->d_chunks, chunks.size() * sizeof(Chunk)), "hipMalloc(chunks)") ||
+        !hip_ok(hipMemcpyAsync(plan->d_recs, recs.data(), recs.size() * sizeof(TensorRec),
+                               hipMemcpyHostToDevice, ctx->stream), "upload recs") ||
+        !hip_ok(hipMemcpyAsync(plan->d_chunks, chunks.data(), chunks.size() * sizeof(Chunk),
+                               hipMemcpyHostToDevice, ctx->stream), "upload chunks") ||
+        !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+        return nullptr;
+    plan->num_chunks = (uint32_t)chunks.size();
+    return plan;
+}
+
+MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req)
+{
+    const int chunk = current_chunk_elements();
+    const uint64_t gen = registry_generation();
+    auto &plans = ctx->plans;
+    for (size_t i = 0; i < plans.size(); i++) {
+        if (plan_matches(*plans[i], req, chunk, gen)) {
+            if (i != 0) std::rotate(plans.begin(), plans.begin() + i, plans.begin() + i + 1);
+            return plans[0].get();
+        }
+    }
+    // Plans of an older registry generation can never match again.
+    for (size_t i = plans.size(); i-- > 0;)
+        if (plans[i]->generation != gen) plans.erase(plans.begin() + i);
+    auto plan = build_plan(ctx, req, chunk, gen);
+    if (!plan) return nullptr;
+    if (plans.size() >= kMaxCachedPlans) plans.pop_back();
+    plans.insert(plans.begin(), std::move(plan));
+    return plans[0].get();
+}
+
+// --------------------------------------------------------------- kernels ----
+template <bool NT, class T>
+__device__ inline T stream_load(const T *p)
+{
+    if (NT) return __builtin_nontemporal_load(p);
+    return *p;
+}
+
+template <bool NT, class T>
+__device__ inline void stream_store(T v, T *p)
+{
+    if (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
+// Applies Rule to `count` elements starting at element `offset` of a tensor.
+// GradT is float or _Float16 (mixed precision: g = float(g16) * inv_scale and
+// an optional fp16 copy of the new weight is emitted).
+template <class Rule, bool NT, bool AMP>
+__device__ inline void process_chunk(const TensorRec &rec, uint64_t offset, uint32_t count,
+                                     const StepParams &prm, float inv_scale)
+{
+    constexpr int NS = Rule::NSTATE;
+    constexpr int NSA = NS > 0 ? NS : 1;
+    float *__restrict__ w = reinterpret_cast<float *>(rec.p[kSlotWeight]) + offset;
+    const float *__restrict__ g32 = nullptr;
+    const _Float16 *__restrict__ g16 = nullptr;
+    _Float16 *__restrict__ w16 = nullptr;
+    if (AMP) {
+        g16 = reinterpret_cast<const _Float16 *>(rec.p[kSlotGrad]) + offset;
+        if (rec.p[kSlotWeight16]) w16 = reinterpret_cast<_Float16 *>(rec.p[kSlotWeight16]) + offset;
+    } else {
+        g32 = reinterpret_cast<const float *>(rec.p[kSlotGrad]) + offset;
+    }
+    float *__restrict__ st[NSA];
+#pragma unroll
+    for (int k = 0; k < NS; k++) st[k] = reinterpret_cast<float *>(rec.p[kSlotState0 + k]) + offset;
+
+    uint32_t done = 0;
+    if (rec.flags & kRecVectorOk) {
+        const uint32_t n4 = count >> 2;
+        floatx4 *w4 = reinterpret_cast<floatx4 *>(w);
+        for (uint32_t base = threadIdx.x; base < n4; base += kBlock * kUnroll) {
+            floatx4 W[kUnroll], G[kUnroll], S[NSA][kUnroll];
+            // all loads first: (2 + NS) * kUnroll independent 16-byte requests per lane
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                const uint32_t i = base + u * kBlock;
+                if (i < n4) {
+                    W[u] = stream_load<NT>(w4 + i);
+                    if (AMP) {
+                        halfx4 h = stream_load<NT>(reinterpret_cast<const halfx4 *>(g16) + i);
+                        G[u] = floatx4{(float)h.x, (float)h.y, (float)h.z, (float)h.w};
+                    } else {
+                        G[u] = stream_load<NT>(reinterpret_cast<const floatx4 *>(g32) + i);
+                    }
+#pragma unroll
+                    for (int k = 0; k < NS; k++)
+                        S[k][u] = stream_load<NT>(reinterpret_cast<const floatx4 *>(st[k]) + i);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                const uint32_t i = base + u * kBlock;
+                if (i < n4) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        float wv = W[u][c];
+                        float gv = G[u][c];
+                        if (AMP) gv = gv * inv_scale;
+                        float sv[NSA];
+#pragma unroll
+                        for (int k = 0; k < NS; k++) sv[k] = S[k][u][c];
+                        Rule::apply(wv, gv, sv, prm);
+                        W[u][c] = wv;
+#pragma unroll
+                        for (int k = 0; k < NS; k++) S[k][u][c] = sv[k];
+                    }
+                    stream_store<NT>(W[u], w4 + i);
+#pragma unroll
+                    for (int k = 0; k < NS; k++)
+                        stream_store<NT>(S[k][u], reinterpret_cast<floatx4 *>(st[k]) + i);
+                    if (AMP && w16) {
+                        halfx4 h = {(_Float16)W[u].x, (_Float16)W[u].y, (_Float16)W[u].z, (_Float16)W[u].w};
+                        stream_store<NT>(h, reinterpret_cast<halfx4 *>(w16) + i);
+                    }
+                }
+            }
+        }
+        done = n4 << 2;
+    }
+    // scalar path: the < 4 element tail, or the whole chunk when a stream is misaligned
+    for (uint32_t i = done + threadIdx.x; i < count; i += kBlock) {
+        float wv = w[i];
+        float gv = AMP ? (float)g16[i] * inv_scale : g32[i];
+        float sv[NSA];
+#pragma unroll
+        for (int k = 0; k < NS; k++) sv[k] = st[k][i];
+        Rule::apply(wv, gv, sv, prm);
+        w[i] = wv;
+#pragma unroll
+        for (int k = 0; k < NS; k++) st[k][i] = sv[k];
+        if (AMP && w16) w16[i] = (_Float16)wv;
+    }
+}
+
+template <class Rule, bool NT>
+__global__ void __launch_bounds__(kBlock)
+multi_tensor_update_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
+                           StepParams prm)
+{
+    const Chunk ch = chunks[blockIdx.x];
+    const TensorRec rec = recs[ch.tensor];
+    process_chunk<Rule, NT, false>(rec, ch.offset, ch.count, prm, 1.0f);
+}
+
+// SGD: a tensor without a momentum buffer takes the vanilla rule.
+template <bool NT>
+__global__ void __launch_bounds__(kBlock)
+multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
+                        StepParams prm)
+{
+    const Chunk ch = chunks[blockIdx.x];
+    const TensorRec rec = recs[ch.tensor];
+    if (prm.momentum > 0.0f && rec.p[kSlotState0] != nullptr)
+        process_chunk<SgdMomentumRule, NT, false>(rec, ch.offset, ch.count, prm, 1.0f);
+    else
+        process_chunk<SgdVanillaRule, NT, false>(rec, ch.offset, ch.count, prm, 1.0f);
+}
+
+// ---- mixed precision ----
+
+// Loss-scale state machine, resident in HBM next to the tensors.
+struct AmpDeviceState {
+    float scale;
+    int growth_tracker;
+    int found_inf;          // set by the check kernel, consumed and cleared by the update kernel
+    unsigned int ticket;    // workgroups of the update kernel that have finished
+    int last_skipped;
+    float growth_factor;
+    float backoff_factor;
+    int growth_interval;
+};
+
+// Phase A: OR over every fp16 gradient element of "exponent field all ones"
+// (+-inf or NaN).  Per lane OR -> wavefront ballot -> one LDS word per wave ->
+// one atomic per workgroup that saw a hit.
+template <bool NT>
+__global__ void __launch_bounds__(kBlock)
+amp_overflow_check_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
+                          AmpDeviceState *__restrict__ state)
+{
+    __shared__ unsigned int wave_hit[kBlock / 64];
+    const Chunk ch = chunks[blockIdx.x];
+    const TensorRec rec = recs[ch.tensor];
+    const unsigned short *g = reinterpret_cast<const unsigned short *>(rec.p[kSlotGrad]) + ch.offset;
+    unsigned int bad = 0;
+    uint32_t done = 0;
+    if (rec.flags & kRecGrad16VectorOk) {
+        const uint32_t n8 = ch.count >> 3;
+        const uintx4 *g8 = reinterpret_cast<const uintx4 *>(g);
+        for (uint32_t base = threadIdx.x; base < n8; base += kBlock * kUnroll) {
+            uintx4 v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                const uint32_t i = base + u * kBlock;
+                v[u] = (i < n8) ? stream_load<NT>(g8 + i) : uintx4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const unsigned int e = v[u][c] & 0x7C007C00u;
+                    bad |= ((e & 0xFFFFu) == 0x7C00u) | ((e >> 16) == 0x7C00u);
+                }
+            }
+        }
+        done = n8 << 3;
+    }
+    for (uint32_t i = done + threadIdx.x; i < ch.count; i += kBlock)
+        bad |= ((g[i] & 0x7C00u) == 0x7C00u);
+
+    const unsigned long long ballot = __ballot(bad != 0);
+    if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = (ballot != 0ull);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned int any = 0;
+#pragma unroll
+        for (int k = 0; k < kBlock / 64; k++) any |= wave_hit[k];
+        if (any) atomicOr(&state->found_inf, 1);
+    }
+}
+
+// Phase B: the Adam update on unscaled gradients, skipped as a whole when the
+// flag is set; the last workgroup to finish advances the loss-scale state.
+template <bool NT>
+__global__ void __launch_bounds__(kBlock)
+amp_adam_update_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
+                       uint32_t num_chunks, StepParams prm, AmpDeviceState *state)
+{
+    const int found = *reinterpret_cast<volatile int *>(&state->found_inf);
+    const float scale = *reinterpret_cast<volatile float *>(&state->scale);
+    if (!found && blockIdx.x < num_chunks) {
+        const float inv_scale = 1.0f / scale;
+        const Chunk ch = chunks[blockIdx.x];
+        const TensorRec rec = recs[ch.tensor];
+        process_chunk<AdamRule, NT, true>(rec, ch.offset, ch.count, prm, inv_scale);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __threadfence();
+        const unsigned int t = atomicAdd(&state->ticket, 1u);
+        if (t == gridDim.x - 1) {
+            // Every other workgroup has read the flag and the scale and finished.
+            float s = scale;
+            int tracker = state->growth_tracker;
+            if (found) {
+                s = s * state->backoff_factor;
+                tracker = 0;
+            } else {
+                tracker += 1;
+                if (tracker == state->growth_interval) {
+                    s = s * state->growth_factor;
+                    tracker = 0;
+                }
+            }
+            state->scale = s;
+            state->growth_tracker = tracker;
+            state->last_skipped = found ? 1 : 0;
+            state->found_inf = 0;
+            state->ticket = 0;
+            __threadfence();
+        }
+    }
+}
+
+// ----------------------------------------------------------- host helpers ----
+static StepParams zero_params()
+{
+    StepParams p;
+    std::memset(&p, 0, sizeof p);
+    return p;
+}
+
+struct Launch {
+    Context *ctx;
+    MultiTensorPlan *plan;
+};
+
+// Resolves the device, takes the context lock, finds the plan.  Returns the
+// entry point's code on failure (hip_error_code for HIP trouble) or 0; when 0
+// and out.plan->num_chunks == 0 there is nothing to launch.
+static int prepare(uintptr_t device, const PlanRequest &req, int hip_error_code, Launch &out,
+                   std::unique_lock<std::mutex> &lock)
+{
+    clear_error();
+    if (device == 0) {
+        set_error("device handle is nil");
+        return -1;
+    }
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (req.num_tensors < 0 || (req.num_tensors > 0 && (!req.sizes || !req.slot[kSlotWeight] ||
+                                                         !req.slot[kSlotGrad]))) {
+        set_error("weight, gradient and size arrays are required");
+        return hip_error_code;
+    }
+    if (!make_current(ctx)) return hip_error_code;
+    lock = std::unique_lock<std::mutex>(ctx->mu);
+    MultiTensorPlan *plan = get_plan(ctx, req);
+    if (!plan) return hip_error_code;
+    if (plan->status != 0) {
+        set_error("a required buffer handle is nil (code %d)", plan->status);
+        return plan->status;
+    }
+    out.ctx = ctx;
+    out.plan = plan;
+    return 0;
+}
+
+template <class Rule>
+static int launch_rule(const Launch &l, const StepParams &prm, int hip_error_code)
+{
+    if (l.plan->num_chunks == 0) return 0;
+    if (current_nontemporal())
+        multi_tensor_update_kernel<Rule, true><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
+            l.plan->d_chunks, l.plan->d_recs, prm);
+    else
+        multi_tensor_update_kernel<Rule, false><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
+            l.plan->d_chunks, l.plan->d_recs, prm);
+    return hip_ok(hipGetLastError(), "update kernel launch") ? 0 : hip_error_code;
+}
+
+static int rmsprop_extra_check(const PlanRequest &req, int i)
+{
+    const bool momentum = (req.variant & 1) != 0, centered = (req.variant & 2) != 0;
+    if (momentum && (!req.slot[kSlotState1] || req.slot[kSlotState1][i] == 0)) return -5;
+    const int ga = momentum ? kSlotState2 : kSlotState1;
+    if (centered && (!req.slot[ga] || req.slot[ga][i] == 0)) return -6;
+    return 0;
+}
+
+static int adam_like_step(int kind, uintptr_t device, uintptr_t *w, uintptr_t *g, uintptr_t *m,
+                          uintptr_t *v, int n, int *sizes, float lr, float beta1, float beta2,
+                          float eps, float wd, int step_count)
+{
+    PlanRequest req{};
+    req.kind = kind;
+    req.num_tensors = n;
+    req.slot[kSlotWeight] = w;
+    req.slot[kSlotGrad] = g;
+    req.slot[kSlotState0] = m;
+    req.slot[kSlotState1] = v;
+    req.sizes = sizes;
+    req.required_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0) | (1u << kSlotState1);
+    req.missing_code = -4;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = prepare(device, req, -6, l, lock)) return rc;
+
+    StepParams p = zero_params();
+    p.lr = lr;
+    p.beta1 = beta1;
+    p.beta2 = beta2;
+    p.one_minus_beta1 = 1.0f - beta1;
+    p.one_minus_beta2 = 1.0f - beta2;
+    p.eps = eps;
+    p.weight_decay = wd;
+    gm_bias_corrections(beta1, beta2, step_count, &p.bc1, &p.bc2);
+    if (kind == kRuleNAdam) {
+        p.mu = gm_nadam_mu_next(beta1, step_count);
+        p.one_minus_mu = 1.0f - p.mu;
+        return launch_rule<NAdamRule>(l, p, -6);
+    }
+    return launch_rule<AdamRule>(l, p, -6);
+}
+
+}  // namespace gm
+
+using namespace gm;
+
+// ================================================================= C ABI ====
+extern "C" {
+
+void gm_bias_corrections(float beta1, float beta2, int step_count, float *bc1, float *bc2)
+{
+    // bridge_optimizer.m:398-399
+    *bc1 = 1.0f - powf(beta1, (float)step_count);
+    *bc2 = 1.0f - powf(beta2, (float)step_count);
+}
+
+float gm_nadam_mu_next(float beta1, int step_count)
+{
+    // bridge_optimizer.m:2066
+    const float exponent = (float)(step_count + 1) * 0.004f;
+    const float decay = powf(0.96f, exponent);
+    const float half_decay = 0.5f * decay;
+    const float one_minus = 1.0f - half_decay;
+    return beta1 * one_minus;
+}
+
+int gm_set_tuning(int chunk_elements, int nontemporal)
+{
+    if (chunk_elements != 0) {
+        if (chunk_elements < 1024 || chunk_elements % 1024 != 0) return -1;
+        g_chunk_elements.store(chunk_elements);
+    } else {
+        g_chunk_elements.store(kDefaultChunkElements);
+    }
+    if (nontemporal >= 0) g_nontemporal.store(nontemporal ? 1 : 0);
+    else g_nontemporal.store(1);
+    return 0;
+}
+
+int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                              uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                              int num_weights, int *buffer_sizes, float learning_rate,
+                              float momentum, float weight_decay, int nesterov, int step_count)
+{
+    (void)step_count;   // unused by the reference as well
+    PlanRequest req{};
+    req.kind = kRuleSGD;
+    req.num_tensors = num_weights;
+    req.slot[kSlotWeight] = weight_buffers;
+    req.slot[kSlotGrad] = gradient_buffers;
+    req.slot[kSlotState0] = momentum > 0.0f ? momentum_buffers : nullptr;
+    req.sizes = buffer_sizes;
+    req.skip_if_zero_mask = (1u << kSlotWeight) | (1u << kSlotGrad);
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = prepare(device, req, -10, l, lock)) return rc;
+    if (l.plan->num_chunks == 0) return 0;
+
+    StepParams p = zero_params();
+    p.lr = learning_rate;
+    p.momentum = momentum;
+    p.weight_decay = weight_decay;
+    p.nesterov = nesterov;
+    if (current_nontemporal())
+        multi_tensor_sgd_kernel<true><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
+            l.plan->d_chunks, l.plan->d_recs, p);
+    else
+        multi_tensor_sgd_kernel<false><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
+            l.plan->d_chunks, l.plan->d_recs, p);
+    return hip_ok(hipGetLastError(), "sgd kernel launch") ? 0 : -10;
+}
+
+int execute_adam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                               uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                               uintptr_t *variance_buffers, int num_weights, int *buffer_sizes,
+                               float learning_rate, float beta1, float beta2, float epsilon,
+                               float weight_decay, int step_count)
+{
+    return adam_like_step(kRuleAdam, device, weight_buffers, gradient_buffers, momentum_buffers,
+                          variance_buffers, num_weights, buffer_sizes, learning_rate, beta1, beta2,
+                          epsilon, weight_decay, step_count);
+}
+
+int execute_adam_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                      uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                                      uintptr_t *variance_buffers, int num_weights,
+                                      int *buffer_sizes, float learning_rate, float beta1,
+                                      float beta2, float epsilon, float weight_decay,
+                                      int step_count, uintptr_t command_pool)
+{
+    if (device == 0) return -1;
+    if (command_pool == 0) return -15;
+    return adam_like_step(kRuleAdam, device, weight_buffers, gradient_buffers, momentum_buffers,
+                          variance_buffers, num_weights, buffer_sizes, learning_rate, beta1, beta2,
+                          epsilon, weight_decay, step_count);
+}
+
+int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                                uintptr_t *variance_buffers, int num_weights, int *buffer_sizes,
+                                float learning_rate, float beta1, float beta2, float epsilon,
+                                float weight_decay, int step_count)
+{
+    return adam_like_step(kRuleNAdam, device, weight_buffers, gradient_buffers, momentum_buffers,
+                          variance_buffers, num_weights, buffer_sizes, learning_rate, beta1, beta2,
+                          epsilon, weight_decay, step_count);
+}
+
+int execute_rmsprop_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                  uintptr_t *gradient_buffers,
+                                  uintptr_t *squared_grad_avg_buffers,
+                                  uintptr_t *momentum_buffers, uintptr_t *gradient_avg_buffers,
+                                  int num_weights, int *buffer_sizes, float learning_rate,
+                                  float alpha, float epsilon, float weight_decay, float momentum,
+                                  bool centered, int step_count)
+{
+    (void)step_count;
+    const bool use_momentum = momentum > 0.0f;
+    PlanRequest req{};
+    req.kind = kRuleRMSProp;
+    req.variant = (use_momentum ? 1 : 0) | (centered ? 2 : 0);
+    req.num_tensors = num_weights;
+    req.slot[kSlotWeight] = weight_buffers;
+    req.slot[kSlotGrad] = gradient_buffers;
+    req.slot[kSlotState0] = squared_grad_avg_buffers;
+    // state order inside the kernel: squared average, [momentum], [gradient average]
+    int next = kSlotState1;
+    if (use_momentum) req.slot[next++] = momentum_buffers;
+    if (centered) req.slot[next++] = gradient_avg_buffers;
+    req.sizes = buffer_sizes;
+    req.required_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0);
+    req.missing_code = -4;
+    req.extra_check = rmsprop_extra_check;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = prepare(device, req, -8, l, lock)) return rc;
+
+    StepParams p = zero_params();
+    p.lr = learning_rate;
+    p.alpha = alpha;
+    p.one_minus_alpha = 1.0f - alpha;
+    p.eps = epsilon;
+    p.weight_decay = weight_decay;
+    p.momentum = momentum;
+    if (use_momentum && centered) return launch_rule<RmsPropRule<true, true>>(l, p, -8);
+    if (use_momentum) return launch_rule<RmsPropRule<true, false>>(l, p, -8);
+    if (centered) return launch_rule<RmsPropRule<false, true>>(l, p, -8);
+    return launch_rule<RmsPropRule<false, false>>(l, p, -8);
+}
+
+int execute_adagrad_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                  uintptr_t *gradient_buffers,
+                                  uintptr_t *squared_grad_avg_buffers, int num_weights,
+                                  int *buffer_sizes, float learning_rate, float epsilon,
+                                  float weight_decay)
+{
+    PlanRequest req{};
+    req.kind = kRuleAdaGrad;
+    req.num_tensors = num_weights;
+    req.slot[kSlotWeight] = weight_buffers;
+    req.slot[kSlotGrad] = gradient_buffers;
+    req.slot[kSlotState0] = squared_grad_avg_buffers;
+    req.sizes = buffer_sizes;
+    req.skip_if_zero_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0);
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = prepare(device, req, -8, l, lock)) return rc;
+    StepParams p = zero_params();
+    p.lr = learning_rate;
+    p.eps = epsilon;
+    p.weight_decay = weight_decay;
+    return launch_rule<AdaGradRule>(l, p, -8);
+}
+
+int execute_adagrad_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                         uintptr_t *gradient_buffers,
+                                         uintptr_t *squared_grad_avg_buffers, int num_weights,
+                                         int *buffer_sizes, float learning_rate, float epsilon,
+                                         float weight_decay, uintptr_t command_pool)
+{
+    (void)command_pool;
+    return execute_adagrad_step_mpsgraph(device, weight_buffers, gradient_buffers,
+                                         squared_grad_avg_buffers, num_weights, buffer_sizes,
+                                         learning_rate, epsilon, weight_decay);
+}
+
+int execute_adadelta_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                   uintptr_t *gradient_buffers,
+                                   uintptr_t *squared_grad_avg_buffers,
+                                   uintptr_t *squared_update_avg_buffers, int num_weights,
+                                   int *buffer_sizes, float rho, float epsilon, float weight_decay)
+{
+    PlanRequest req{};
+    req.kind = kRuleAdaDelta;
+    req.num_tensors = num_weights;
+    req.slot[kSlotWeight] = weight_buffers;
+    req.slot[kSlotGrad] = gradient_buffers;
+    req.slot[kSlotState0] = squared_grad_avg_buffers;
+    req.slot[kSlotState1] = squared_update_avg_buffers;
+    req.sizes = buffer_sizes;
+    req.skip_if_zero_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0) |
+                            (1u << kSlotState1);
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = prepare(device, req, -8, l, lock)) return rc;
+    StepParams p = zero_params();
+    p.rho = rho;
+    p.one_minus_rho = 1.0f - rho;
+    p.eps = epsilon;
+    p.weight_decay = weight_decay;
+    return launch_rule<AdaDeltaRule>(l, p, -8);
+}
+
+int execute_adadelta_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                          uintptr_t *gradient_buffers,
+                                          uintptr_t *squared_grad_avg_buffers,
+                                          uintptr_t *squared_update_avg_buffers, int num_weights,
+                                          int *buffer_sizes, float rho, float epsilon,
+                                          float weight_decay, uintptr_t command_pool)
+{
+    (void)command_pool;
+    return execute_adadelta_step_mpsgraph(device, weight_buffers, gradient_buffers,
+                                          squared_grad_avg_buffers, squared_update_avg_buffers,
+                                          num_weights, buffer_sizes, rho, epsilon, weight_decay);
+}
+
+// ---------------------------------------------------------- mixed precision --
+struct AmpState {
+    uint64_t magic;
+    Context *ctx;
+    AmpDeviceState *d_state;
+    AmpDeviceState *h_pinned;
+};
+static const uint64_t kAmpMagic = 0x676D5F616D705F73ull;   // "gm_amp_s"
+
+static AmpState *amp_from_handle(uintptr_t h)
+{
+    if (h == 0) return nullptr;
+    auto *s = reinterpret_cast<AmpState *>(h);
+    return s->magic == kAmpMagic ? s : nullptr;
+}
+
+static bool amp_upload(AmpState *s)
+{
+    return hip_ok(hipMemcpyAsync(s->d_state, s->h_pinned, sizeof(AmpDeviceState),
+                                 hipMemcpyHostToDevice, s->ctx->stream), "amp state upload") &&
+           hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize");
+}
+
+static bool amp_download(AmpState *s)
+{
+    return hip_ok(hipMemcpyAsync(s->h_pinned, s->d_state, sizeof(AmpDeviceState),
+                                 hipMemcpyDeviceToHost, s->ctx->stream), "amp state download") &&
+           hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize");
+}
+
+uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_factor,
+                              float backoff_factor, int growth_interval)
+{
+    clear_error();
+    if (device == 0) return 0;
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return 0;
+    auto *s = new AmpState{kAmpMagic, ctx, nullptr, nullptr};
+    if (!hip_ok(hipMalloc(&s->d_state, sizeof(AmpDeviceState)), "hipMalloc(amp state)") ||
+        !hip_ok(hipHostMalloc(&s->h_pinned, sizeof(AmpDeviceState), hipHostMallocDefault),
+                "hipHostMalloc(amp state)")) {
+        if (s->d_state) (void)hipFree(s->d_state);
+        delete s;
+        return 0;
+    }
+    *s->h_pinned = AmpDeviceState{init_scale, 0, 0, 0u, 0, growth_factor, backoff_factor, growth_interval};
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    if (!amp_upload(s)) {
+        (void)hipFree(s->d_state);
+        (void)hipHostFree(s->h_pinned);
+        delete s;
+        return 0;
+    }
+    return reinterpret_cast<uintptr_t>(s);
+}
+
+void gm_amp_state_destroy(uintptr_t amp_state)
+{
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return;
+    make_current(s->ctx);
+    s->magic = 0;
+    (void)hipFree(s->d_state);
+    (void)hipHostFree(s->h_pinned);
+    delete s;
+}
+
+int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker)
+{
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    if (scale) *scale = s->h_pinned->scale;
+    if (growth_tracker) *growth_tracker = s->h_pinned->growth_tracker;
+    return 0;
+}
+
+int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
+{
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    s->h_pinned->scale = scale;
+    s->h_pinned->growth_tracker = growth_tracker;
+    return amp_upload(s) ? 0 : -6;
+}
+
+int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
+                          uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                          uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                          int num_weights, int *buffer_sizes, float learning_rate, float beta1,
+                          float beta2, float epsilon, float weight_decay, int step_count,
+                          uintptr_t amp_state, int *skipped, float *scale_out,
+                          int *growth_tracker_out)
+{
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    PlanRequest req{};
+    req.kind = kRuleAdamAMP;
+    req.num_tensors = num_weights;
+    req.slot[kSlotWeight] = weight_buffers;
+    req.slot[kSlotGrad] = gradient16_buffers;
+    req.slot[kSlotState0] = momentum_buffers;
+    req.slot[kSlotState1] = variance_buffers;
+    req.slot[kSlotWeight16] = weight16_buffers;
+    req.sizes = buffer_sizes;
+    req.required_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0) | (1u << kSlotState1);
+    req.missing_code = -4;
+    req.half_mask = (1u << kSlotGrad) | (1u << kSlotWeight16);
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = prepare(device, req, -6, l, lock)) return rc;
+
+    StepParams p = zero_params();
+    p.lr = learning_rate;
+    p.beta1 = beta1;
+    p.beta2 = beta2;
+    p.one_minus_beta1 = 1.0f - beta1;
+    p.one_minus_beta2 = 1.0f - beta2;
+    p.eps = epsilon;
+    p.weight_decay = weight_decay;
+    gm_bias_corrections(beta1, beta2, step_count, &p.bc1, &p.bc2);
+
+    const uint32_t chunks = l.plan->num_chunks;
+    const uint32_t grid = chunks > 0 ? chunks : 1;
+    hipStream_t st = l.ctx->stream;
+    if (current_nontemporal()) {
+        if (chunks > 0)
+            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs,
+                                                                      amp->d_state);
+        amp_adam_update_kernel<true><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, chunks,
+                                                             p, amp->d_state);
+    } else {
+        if (chunks > 0)
+            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs,
+                                                                       amp->d_state);
+        amp_adam_update_kernel<false><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, chunks,
+                                                              p, amp->d_state);
+    }
+    if (!hip_ok(hipGetLastError(), "mixed-precision kernel launch")) return -6;
+    if (!amp_download(amp)) return -6;
+    if (skipped) *skipped = amp->h_pinned->last_skipped;
+    if (scale_out) *scale_out = amp->h_pinned->scale;
+    if (growth_tracker_out) *growth_tracker_out = amp->h_pinned->growth_tracker;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+// Multi-tensor launch plan: the device-side tables one update launch walks.
+//
+// A step over a parameter list is ONE kernel launch.  The host flattens the
+// list into fixed-size chunks; workgroup b processes chunk b.  Two small tables
+// live in HBM and are rebuilt only when the caller's handles change:
+//
+//   TensorRec recs[num_tensors]   base addresses of every stream of a tensor
+//   Chunk     chunks[num_chunks]  {tensor index, element offset, element count}
+//
+// Both are read with wave-uniform (scalar) loads, so they cost one cache line
+// per workgroup against >= 100 KB of streamed data.
+#pragma once
+
+#include "gm_context.hpp"
+
+namespace gm {
+
+// Stream slots of a tensor record.
+enum : int {
+    kSlotWeight = 0,
+    kSlotGrad = 1,     // fp32, or fp16 for the mixed-precision step
+    kSlotState0 = 2,
+    kSlotState1 = 3,
+    kSlotState2 = 4,
+    kSlotWeight16 = 5,
+    kNumSlots = 6,
+};
+
+enum : uint32_t {
+    kRecVectorOk = 1u,       // every used stream is aligned for 16-byte (fp32) / 8-byte (fp16) lanes
+    kRecGrad16VectorOk = 2u, // the fp16 gradient is 16-byte aligned (overflow-check kernel)
+};
+
+struct TensorRec {
+    void *p[kNumSlots];
+    uint32_t flags;
+    uint32_t pad;
+};
+static_assert(sizeof(TensorRec) == 56, "TensorRec layout");
+
+struct Chunk {
+    uint32_t tensor;
+    uint32_t count;     // elements in this chunk (<= chunk_elements)
+    uint64_t offset;    // first element, multiple of chunk_elements
+};
+static_assert(sizeof(Chunk) == 16, "Chunk layout");
+
+// Which update rule a plan (and its validation) was built for.
+enum RuleKind : int {
+    kRuleSGD = 0,
+    kRuleAdam,
+    kRuleRMSProp,
+    kRuleAdaGrad,
+    kRuleAdaDelta,
+    kRuleNAdam,
+    kRuleAdamAMP,
+};
+
+struct MultiTensorPlan {
+    // ---- key ----
+    int kind = 0;
+    int variant = 0;             // rule-specific bits that change validation (e.g. which optional states are on)
+    int num_tensors = 0;
+    int chunk_elements = 0;
+    uint64_t generation = 0;
+    std::vector<uintptr_t> handles;   // kNumSlots * num_tensors, slot-major
+    std::vector<int> sizes;
+    // ---- result ----
+    int status = 0;              // validation result: 0 or the entry point's error code
+    TensorRec *d_recs = nullptr;
+    Chunk *d_chunks = nullptr;
+    uint32_t num_chunks = 0;
+    uint64_t total_elements = 0;
+    ~MultiTensorPlan();
+};
+
+// What an entry point hands to the planner.  slot[k] is the caller's handle
+// array for stream k (nullptr = stream unused by this rule: all zeros).
+struct PlanRequest {
+    int kind;
+    int variant;
+    int num_tensors;
+    const uintptr_t *slot[kNumSlots];
+    const int *sizes;            // bytes of the fp32 weight tensor
+    uint32_t required_mask;      // slots whose handle must be non-zero ...
+    int missing_code;            // ... else the step fails with this code (0: skip that tensor instead)
+    uint32_t skip_if_zero_mask;  // slots whose zero handle makes the tensor be skipped (when missing_code == 0)
+    uint32_t half_mask;          // slots holding fp16 elements (length and alignment checks)
+    // Optional extra per-tensor check run on a cache miss; returns a non-zero
+    // error code to fail the step.
+    int (*extra_check)(const PlanRequest &req, int tensor);
+};
+
+// Returns the cached plan for this request or builds one (under ctx->mu, which
+// the caller holds).  nullptr on a HIP failure (error already recorded).
+MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req);
+
+// Elements per workgroup chunk currently in force (tunable for sweeps).
+int current_chunk_elements();
+// Whether streaming accesses carry the non-temporal hint.
+bool current_nontemporal();
+
+}  // namespace gm

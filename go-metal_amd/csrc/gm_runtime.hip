@@ -1,0 +1,515 @@
+// Device, queue and buffer entry points of the C ABI (the HIP counterpart of
+// cgo_bridge/bridge_memory.m and the device / queue part of bridge_device.m),
+// plus the measurement helpers.
+#include "gm_context.hpp"
+#include "gm_plan.hpp"
+
+#include "../../include/gometal_hip.h"
+
+#include <hip/hip_fp16.h>
+
+#include <cstring>
+
+namespace gm {
+
+// ---------------------------------------------------------------- errors ----
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+}
+
+void clear_error() { g_error[0] = '\0'; }
+
+bool hip_ok(hipError_t e, const char *what)
+{
+    if (e == hipSuccess) return true;
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return false;
+}
+
+// --------------------------------------------------------------- context ----
+Context::~Context() = default;
+
+static Context *g_ctx = nullptr;
+static std::once_flag g_ctx_once;
+
+Context *default_context()
+{
+    std::call_once(g_ctx_once, [] {
+        int count = 0;
+        if (hipGetDeviceCount(&count) != hipSuccess || count < 1) {
+            set_error("no HIP device is visible");
+            return;
+        }
+        auto *ctx = new Context();   // lives until the process ends
+        ctx->device_id = 0;
+        if (!hip_ok(hipSetDevice(0), "hipSetDevice") ||
+            !hip_ok(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking), "hipStreamCreate") ||
+            !hip_ok(hipEventCreate(&ctx->ev_start), "hipEventCreate") ||
+            !hip_ok(hipEventCreate(&ctx->ev_stop), "hipEventCreate")) {
+            delete ctx;
+            return;
+        }
+        ctx->usable = true;
+        g_ctx = ctx;
+    });
+    return g_ctx;
+}
+
+Context *resolve_device(uintptr_t device)
+{
+    if (device == 0) return nullptr;
+    return default_context();
+}
+
+bool make_current(Context *ctx) { return hip_ok(hipSetDevice(ctx->device_id), "hipSetDevice"); }
+
+// -------------------------------------------------------------- registry ----
+static std::mutex g_reg_mu;
+static std::unordered_map<uintptr_t, size_t> g_reg;
+static std::atomic<uint64_t> g_reg_generation{1};
+
+void registry_add(uintptr_t buffer, size_t bytes)
+{
+    std::lock_guard<std::mutex> lk(g_reg_mu);
+    g_reg[buffer] = bytes;
+}
+
+void registry_remove(uintptr_t buffer)
+{
+    std::lock_guard<std::mutex> lk(g_reg_mu);
+    g_reg.erase(buffer);
+    g_reg_generation.fetch_add(1);
+}
+
+size_t registry_length(uintptr_t buffer)
+{
+    std::lock_guard<std::mutex> lk(g_reg_mu);
+    auto it = g_reg.find(buffer);
+    return it == g_reg.end() ? 0 : it->second;
+}
+
+uint64_t registry_generation() { return g_reg_generation.load(); }
+
+// --------------------------------------------------------------- kernels ----
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+// fp32 -> fp16, round to nearest even (v_cvt_f16_f32); 4 elements per lane,
+// scalar tail.
+__global__ void __launch_bounds__(256)
+convert_f32_to_f16_kernel(const float *__restrict__ src, __half *__restrict__ dst, size_t n)
+{
+    const size_t n4 = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        floatx4 x = reinterpret_cast<const floatx4 *>(src)[i];
+        __half2 lo = __halves2half2(__float2half_rn(x.x), __float2half_rn(x.y));
+        __half2 hi = __halves2half2(__float2half_rn(x.z), __float2half_rn(x.w));
+        uint2 packed;
+        packed.x = *reinterpret_cast<unsigned int *>(&lo);
+        packed.y = *reinterpret_cast<unsigned int *>(&hi);
+        reinterpret_cast<uint2 *>(dst)[i] = packed;
+    }
+    if (blockIdx.x == 0) {
+        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += blockDim.x) dst[i] = __float2half_rn(src[i]);
+    }
+}
+
+__global__ void __launch_bounds__(256)
+convert_f16_to_f32_kernel(const __half *__restrict__ src, float *__restrict__ dst, size_t n)
+{
+    const size_t n4 = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        uint2 packed = reinterpret_cast<const uint2 *>(src)[i];
+        __half2 lo = *reinterpret_cast<__half2 *>(&packed.x);
+        __half2 hi = *reinterpret_cast<__half2 *>(&packed.y);
+        floatx4 y;
+        y.x = __low2float(lo);
+        y.y = __high2float(lo);
+        y.z = __low2float(hi);
+        y.w = __high2float(hi);
+        reinterpret_cast<floatx4 *>(dst)[i] = y;
+    }
+    if (blockIdx.x == 0) {
+        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += blockDim.x) dst[i] = __half2float(src[i]);
+    }
+}
+
+// Zero fill: 16-byte stores, byte tail.  (A kernel rather than hipMemsetAsync, so
+// the entry point stays safe to record into a HIP graph.)
+__global__ void __launch_bounds__(256)
+zero_kernel(unsigned char *__restrict__ dst, size_t bytes)
+{
+    const size_t n16 = bytes / 16;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const uintx4 z = {0u, 0u, 0u, 0u};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+        reinterpret_cast<uintx4 *>(dst)[i] = z;
+    if (blockIdx.x == 0) {
+        for (size_t i = n16 * 16 + threadIdx.x; i < bytes; i += blockDim.x) dst[i] = 0;
+    }
+}
+
+// 16 bytes per lane, 4 loads in flight per lane.
+__global__ void __launch_bounds__(256)
+copy_probe_kernel(const uintx4 *__restrict__ src, uintx4 *__restrict__ dst, size_t n16)
+{
+    const size_t base = (size_t)blockIdx.x * (256 * 4) + threadIdx.x;
+    uintx4 r[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n16) r[u] = __builtin_nontemporal_load(&src[i]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n16) __builtin_nontemporal_store(r[u], &dst[i]);
+    }
+}
+
+__device__ inline uint64_t splitmix64(uint64_t x)
+{
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+// One Box-Muller pair per two consecutive elements.
+__device__ inline void normal_pair(uint64_t seed, size_t pair_index, float &a, float &b)
+{
+    uint64_t r = splitmix64(seed ^ (0xD1B54A32D192ED03ull * (uint64_t)(pair_index + 1)));
+    float u1 = ((float)(uint32_t)(r >> 40) + 1.0f) * (1.0f / 16777216.0f);   // (0, 1]
+    float u2 = (float)(uint32_t)((r >> 8) & 0xFFFFFFu) * (1.0f / 16777216.0f);
+    float rad = sqrtf(-2.0f * logf(u1));
+    float s, c;
+    sincosf(6.28318530717958647692f * u2, &s, &c);
+    a = rad * c;
+    b = rad * s;
+}
+
+template <bool HALF>
+__global__ void __launch_bounds__(256)
+fill_normal_kernel(void *__restrict__ dst, size_t n, uint64_t seed, float mean, float std, float scale)
+{
+    const size_t pairs = (n + 1) / 2;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += stride) {
+        float a, b;
+        normal_pair(seed, p, a, b);
+        a = a * std + mean;
+        b = b * std + mean;
+        const size_t i = 2 * p;
+        if (HALF) {
+            __half *d = reinterpret_cast<__half *>(dst);
+            d[i] = __float2half_rn(a * scale);
+            if (i + 1 < n) d[i + 1] = __float2half_rn(b * scale);
+        } else {
+            float *d = reinterpret_cast<float *>(dst);
+            d[i] = a;
+            if (i + 1 < n) d[i + 1] = b;
+        }
+    }
+}
+
+static unsigned int grid_for(size_t work_items, unsigned int block, unsigned int max_blocks)
+{
+    size_t blocks = (work_items + block - 1) / block;
+    if (blocks < 1) blocks = 1;
+    if (blocks > max_blocks) blocks = max_blocks;
+    return (unsigned int)blocks;
+}
+
+}  // namespace gm
+
+using namespace gm;
+
+// ================================================================= C ABI ====
+extern "C" {
+
+const char *gm_last_error(void) { return g_error; }
+
+uintptr_t create_metal_device(void)
+{
+    Context *ctx = default_context();
+    if (!ctx) return 0;
+    ctx->refs.fetch_add(1);
+    return reinterpret_cast<uintptr_t>(ctx);
+}
+
+void destroy_metal_device(uintptr_t device)
+{
+    Context *ctx = g_ctx;
+    if (device == 0 || !ctx || reinterpret_cast<uintptr_t>(ctx) != device) return;
+    // The context outlives every handle: pooled buffers and cached plans reached
+    // through another handle must stay valid.  Only the count is dropped.
+    if (ctx->refs.load() > 0) ctx->refs.fetch_sub(1);
+}
+
+struct CommandQueue {
+    uint64_t magic;
+    Context *ctx;
+};
+static const uint64_t kQueueMagic = 0x676D5F7175657565ull;   // "gm_queue"
+
+uintptr_t create_command_queue(uintptr_t device)
+{
+    if (device == 0) return 0;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return 0;
+    return reinterpret_cast<uintptr_t>(new CommandQueue{kQueueMagic, ctx});
+}
+
+void release_command_queue(uintptr_t command_queue)
+{
+    if (command_queue == 0) return;
+    auto *q = reinterpret_cast<CommandQueue *>(command_queue);
+    if (q->magic != kQueueMagic) return;
+    q->magic = 0;
+    delete q;
+}
+
+uintptr_t allocate_metal_buffer(uintptr_t device, int size, int device_type)
+{
+    (void)device_type;
+    if (device == 0 || size <= 0) return 0;
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return 0;
+    const size_t aligned = ((size_t)size + 15) / 16 * 16;
+    void *p = nullptr;
+    if (!hip_ok(hipMalloc(&p, aligned), "hipMalloc")) return 0;
+    registry_add(reinterpret_cast<uintptr_t>(p), aligned);
+    return reinterpret_cast<uintptr_t>(p);
+}
+
+void deallocate_metal_buffer(uintptr_t buffer)
+{
+    if (buffer == 0) return;
+    if (registry_length(buffer) == 0) return;   // not ours (or already freed): leave it alone
+    registry_remove(buffer);
+    Context *ctx = default_context();
+    if (ctx) make_current(ctx);
+    (void)hipFree(reinterpret_cast<void *>(buffer));   // hipFree waits for work in flight
+}
+
+size_t gm_buffer_length(uintptr_t buffer) { return registry_length(buffer); }
+
+int zero_metal_buffer(uintptr_t device, uintptr_t buffer, int size)
+{
+    if (device == 0 || buffer == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return -5;
+    if (size <= 0) return 0;
+    const size_t len = registry_length(buffer);
+    if (len != 0 && (size_t)size > len) {
+        set_error("zero of %d bytes exceeds the %zu-byte buffer", size, len);
+        return -5;
+    }
+    const unsigned int grid = grid_for(((size_t)size + 15) / 16, 256, 1u << 16);
+    zero_kernel<<<grid, 256, 0, ctx->stream>>>(reinterpret_cast<unsigned char *>(buffer), (size_t)size);
+    if (!hip_ok(hipGetLastError(), "zero kernel launch")) return -5;
+    return 0;
+}
+
+int zero_metal_buffer_mpsgraph(uintptr_t device, uintptr_t buffer, int size)
+{
+    return zero_metal_buffer(device, buffer, size);
+}
+
+int copy_data_to_metal_buffer(uintptr_t buffer, void *data, int size)
+{
+    if (buffer == 0 || data == nullptr || size <= 0) return -1;
+    Context *ctx = default_context();
+    if (!ctx || !make_current(ctx)) return -4;
+    // Pageable source: the call returns once the host range has been consumed,
+    // and the copy is ordered after earlier work on the stream.
+    if (!hip_ok(hipMemcpyAsync(reinterpret_cast<void *>(buffer), data, (size_t)size,
+                               hipMemcpyHostToDevice, ctx->stream), "hipMemcpyAsync(H2D)") ||
+        !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+        return -4;
+    return 0;
+}
+
+int copy_float32_array_to_metal_buffer(uintptr_t buffer, float *data, int num_elements)
+{
+    if (buffer == 0 || data == nullptr || num_elements <= 0) return -1;
+    if ((size_t)num_elements * sizeof(float) > 0x7FFFFFFFull) return -1;
+    return copy_data_to_metal_buffer(buffer, data, num_elements * (int)sizeof(float));
+}
+
+int copy_int32_array_to_metal_buffer(uintptr_t buffer, int *data, int num_elements)
+{
+    if (buffer == 0 || data == nullptr || num_elements <= 0) return -1;
+    if ((size_t)num_elements * sizeof(int) > 0x7FFFFFFFull) return -1;
+    return copy_data_to_metal_buffer(buffer, data, num_elements * (int)sizeof(int));
+}
+
+static int copy_from_buffer(uintptr_t buffer, void *data, size_t bytes)
+{
+    Context *ctx = default_context();
+    if (!ctx || !make_current(ctx)) return -4;
+    if (!hip_ok(hipMemcpyAsync(data, reinterpret_cast<void *>(buffer), bytes, hipMemcpyDeviceToHost,
+                               ctx->stream), "hipMemcpyAsync(D2H)") ||
+        !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+        return -4;
+    return 0;
+}
+
+int copy_metal_buffer_to_float32_array(uintptr_t buffer, float *data, int num_elements)
+{
+    if (buffer == 0 || data == nullptr || num_elements <= 0) return -1;
+    return copy_from_buffer(buffer, data, (size_t)num_elements * sizeof(float));
+}
+
+int copy_metal_buffer_to_int32_array(uintptr_t buffer, int *data, int num_elements)
+{
+    if (buffer == 0 || data == nullptr || num_elements <= 0) return -1;
+    return copy_from_buffer(buffer, data, (size_t)num_elements * sizeof(int));
+}
+
+int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, int num_dims,
+                        int src_type, int dst_type, uintptr_t device)
+{
+    if (src_buffer == 0 || dst_buffer == 0 || shape == nullptr || num_dims <= 0) return -1;
+    if (device == 0) return -2;
+    size_t total = 1;
+    for (int i = 0; i < num_dims; i++) {
+        if (shape[i] < 0) return -1;
+        total *= (size_t)shape[i];
+    }
+    const bool to_half = (src_type == 0 && dst_type == 2);
+    const bool to_float = (src_type == 2 && dst_type == 0);
+    if (!to_half && !to_float) return -3;
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return -4;
+    if (total == 0) return 0;
+    const unsigned int grid = grid_for((total + 3) / 4, 256, 1u << 20);
+    if (to_half)
+        convert_f32_to_f16_kernel<<<grid, 256, 0, ctx->stream>>>(
+            reinterpret_cast<const float *>(src_buffer), reinterpret_cast<__half *>(dst_buffer), total);
+    else
+        convert_f16_to_f32_kernel<<<grid, 256, 0, ctx->stream>>>(
+            reinterpret_cast<const __half *>(src_buffer), reinterpret_cast<float *>(dst_buffer), total);
+    if (!hip_ok(hipGetLastError(), "convert kernel launch")) return -4;
+    return 0;
+}
+
+int copy_buffer_to_buffer_sync(uintptr_t src_buffer, uintptr_t dst_buffer, int src_offset,
+                               int dst_offset, int size)
+{
+    if (src_buffer == 0 || dst_buffer == 0) return -1;
+    if (size <= 0 || src_offset < 0 || dst_offset < 0) return -2;
+    const size_t src_len = registry_length(src_buffer);
+    const size_t dst_len = registry_length(dst_buffer);
+    if (src_len != 0 && (size_t)src_offset + (size_t)size > src_len) return -4;
+    if (dst_len != 0 && (size_t)dst_offset + (size_t)size > dst_len) return -5;
+    Context *ctx = default_context();
+    if (!ctx || !make_current(ctx)) return -10;
+    if (!hip_ok(hipMemcpyAsync(reinterpret_cast<char *>(dst_buffer) + dst_offset,
+                               reinterpret_cast<const char *>(src_buffer) + src_offset, (size_t)size,
+                               hipMemcpyDeviceToDevice, ctx->stream), "hipMemcpyAsync(D2D)") ||
+        !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+        return -10;
+    return 0;
+}
+
+int gm_synchronize(uintptr_t device)
+{
+    if (device == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (!make_current(ctx) || !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+        return -10;
+    return 0;
+}
+
+int gm_timer_start(uintptr_t device)
+{
+    if (device == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (!make_current(ctx) || !hip_ok(hipEventRecord(ctx->ev_start, ctx->stream), "hipEventRecord"))
+        return -10;
+    return 0;
+}
+
+float gm_timer_stop(uintptr_t device)
+{
+    if (device == 0) return -1.0f;
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return -1.0f;
+    float ms = -1.0f;
+    if (!hip_ok(hipEventRecord(ctx->ev_stop, ctx->stream), "hipEventRecord") ||
+        !hip_ok(hipEventSynchronize(ctx->ev_stop), "hipEventSynchronize") ||
+        !hip_ok(hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop), "hipEventElapsedTime"))
+        return -1.0f;
+    return ms;
+}
+
+static int fill_normal(uintptr_t device, uintptr_t buffer, size_t n, uint64_t seed, float mean,
+                       float std, float scale, bool half)
+{
+    if (device == 0) return -1;
+    if (buffer == 0) return -4;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (!make_current(ctx)) return -10;
+    if (n == 0) return 0;
+    const size_t len = registry_length(buffer);
+    if (len != 0 && n * (half ? 2 : 4) > len) {
+        set_error("fill of %zu elements exceeds the %zu-byte buffer", n, len);
+        return -5;
+    }
+    const unsigned int grid = grid_for((n + 1) / 2, 256, 1u << 16);
+    if (half)
+        fill_normal_kernel<true><<<grid, 256, 0, ctx->stream>>>(reinterpret_cast<void *>(buffer), n,
+                                                                 seed, mean, std, scale);
+    else
+        fill_normal_kernel<false><<<grid, 256, 0, ctx->stream>>>(reinterpret_cast<void *>(buffer), n,
+                                                                  seed, mean, std, scale);
+    return hip_ok(hipGetLastError(), "fill kernel launch") ? 0 : -10;
+}
+
+int gm_fill_normal_f32(uintptr_t device, uintptr_t buffer, size_t num_elements, uint64_t seed,
+                       float mean, float std)
+{
+    return fill_normal(device, buffer, num_elements, seed, mean, std, 1.0f, false);
+}
+
+int gm_fill_normal_f16(uintptr_t device, uintptr_t buffer, size_t num_elements, uint64_t seed,
+                       float mean, float std, float scale)
+{
+    return fill_normal(device, buffer, num_elements, seed, mean, std, scale, true);
+}
+
+int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, size_t bytes)
+{
+    if (device == 0) return -1;
+    if (dst_buffer == 0 || src_buffer == 0) return -4;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (!make_current(ctx)) return -10;
+    const size_t src_len = registry_length(src_buffer), dst_len = registry_length(dst_buffer);
+    if ((src_len != 0 && bytes > src_len) || (dst_len != 0 && bytes > dst_len) || bytes % 16 != 0) {
+        set_error("copy probe of %zu bytes does not fit (src %zu, dst %zu) or is not a multiple of 16",
+                  bytes, src_len, dst_len);
+        return -5;
+    }
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return 0;
+    const size_t blocks = (n16 + 1023) / 1024;
+    if (blocks > 0x7FFFFFFFull) return -5;
+    copy_probe_kernel<<<(unsigned int)blocks, 256, 0, ctx->stream>>>(
+        reinterpret_cast<const uintx4 *>(src_buffer), reinterpret_cast<uintx4 *>(dst_buffer), n16);
+    return hip_ok(hipGetLastError(), "copy probe launch") ? 0 : -10;
+}
+
+}  // extern "C"

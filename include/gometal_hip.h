@@ -1,0 +1,251 @@
+/*
+ * C ABI of libgometal_hip.so: the MI355X (gfx950) replacement for the part of
+ * go-metal's Objective-C bridge that the `optimizer` package reaches:
+ * cgo_bridge/bridge_optimizer.m (update rules), cgo_bridge/bridge_memory.m
+ * (buffers) and the device / queue subset of cgo_bridge/bridge_device.m.
+ *
+ * Every function in the first part keeps the name, argument order, argument
+ * meaning and return-code convention of the C prototype that
+ * cgo_bridge/bridge.go declares in its cgo preamble, so the Go wrappers in
+ * bridge.go bind to this library unchanged.  Handles are opaque uintptr_t:
+ * a buffer handle IS the device address of the allocation (kernels take it
+ * without indirection); a device handle is a pointer to a process-lifetime
+ * context; 0 is the nil handle everywhere.  Return 0 = success, negative =
+ * error (per-function tables below).  No function throws or aborts.
+ *
+ * Ordering: all work is enqueued on one HIP stream per device context.  The
+ * update entry points return after enqueueing; every entry point that hands
+ * data to the host (copy_metal_buffer_to_*), and copy_buffer_to_buffer_sync,
+ * synchronise that stream before returning, so the host observes the same
+ * values it would after the reference's blocking calls.
+ *
+ * Sizes: buffer_sizes[] are BYTES of the fp32 weight tensor, as in the
+ * reference (numel = size / 4).  They cross this ABI as C int, so one tensor
+ * is limited to 2 GiB - 1 (cgo_bridge/bridge.go:920, 1003).
+ */
+#ifndef GOMETAL_HIP_H
+#define GOMETAL_HIP_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* Device and queue.  cgo_bridge/bridge_device.m:87-107, 901-925;            */
+/* prototypes cgo_bridge/bridge.go:57-60, 247-248.                           */
+/* ------------------------------------------------------------------------ */
+
+/* Returns a handle to the context of HIP device 0 (created on first use, kept
+ * until the process ends, reference counted), or 0 when no GPU is usable.
+ * All handles alias the same GPU, as MTLCreateSystemDefaultDevice does. */
+uintptr_t create_metal_device(void);
+/* Drops one reference.  Buffers, streams and pooled memory reachable through
+ * other handles stay valid (memory/manager.go:246-250 keeps the first handle). */
+void destroy_metal_device(uintptr_t device);
+/* 0 when device is 0 (bridge_device.m:903-906); else an ordering token for the
+ * context's stream. */
+uintptr_t create_command_queue(uintptr_t device);
+void release_command_queue(uintptr_t command_queue);
+
+/* ------------------------------------------------------------------------ */
+/* Buffers.  cgo_bridge/bridge_memory.m; prototypes bridge.go:75-77, 110-137. */
+/* ------------------------------------------------------------------------ */
+
+/* bridge_memory.m:4-42.  size <= 0 or device 0 -> 0.  The length is rounded up
+ * to 16 bytes (:28); the address is 256-byte aligned.  device_type 0=CPU
+ * 1=GPU 2=PersistentGPU (bridge.go:623-629) all map to HBM. */
+uintptr_t allocate_metal_buffer(uintptr_t device, int size, int device_type);
+/* bridge_memory.m:45-55.  0 is ignored. */
+void deallocate_metal_buffer(uintptr_t buffer);
+/* bridge_memory.m:163-188.  -1: nil device or buffer; -5: HIP error. */
+int zero_metal_buffer(uintptr_t device, uintptr_t buffer, int size);
+/* bridge_memory.m:58-160; same effect as zero_metal_buffer here. */
+int zero_metal_buffer_mpsgraph(uintptr_t device, uintptr_t buffer, int size);
+/* bridge_memory.m:191-218.  -1: nil buffer / NULL data / size <= 0; -4: HIP error. */
+int copy_data_to_metal_buffer(uintptr_t buffer, void *data, int size);
+/* bridge_memory.m:221-258.  -1: nil / NULL / n <= 0. */
+int copy_float32_array_to_metal_buffer(uintptr_t buffer, float *data, int num_elements);
+int copy_int32_array_to_metal_buffer(uintptr_t buffer, int *data, int num_elements);
+/* bridge_memory.m:261-320.  Synchronises the stream first.  -1 / -4 as above. */
+int copy_metal_buffer_to_float32_array(uintptr_t buffer, float *data, int num_elements);
+int copy_metal_buffer_to_int32_array(uintptr_t buffer, int *data, int num_elements);
+/* bridge_memory.m:323-423.  Element count = product of shape[0..num_dims).
+ * Type codes from memory/tensor.go:12-17: Float32 = 0, Float16 = 2.
+ * fp32->fp16 rounds to nearest even and overflows to +-inf; fp16->fp32 is
+ * exact.  -1: nil buffers / NULL shape / num_dims <= 0; -2: nil device;
+ * -3: any pair other than 0->2 or 2->0; -4: HIP error. */
+int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, int num_dims,
+                        int src_type, int dst_type, uintptr_t device);
+/* bridge_memory.m:504-592.  -1: nil handle; -2: size <= 0 or negative offset;
+ * -4 / -5: source / destination range exceeds the allocation; -10: HIP error. */
+int copy_buffer_to_buffer_sync(uintptr_t src_buffer, uintptr_t dst_buffer, int src_offset,
+                               int dst_offset, int size);
+
+/* ------------------------------------------------------------------------ */
+/* Optimizer steps.  cgo_bridge/bridge_optimizer.h; prototypes                */
+/* bridge.go:79-123, 277-413.  Arrays have num_weights entries of buffer      */
+/* handles; they are read during the call and not retained.  Weights and      */
+/* states are updated in place; gradients are read only.                      */
+/* Common codes: -1 device 0 (checked first, nothing else touched);           */
+/* -3 no usable GPU stream; others per function.  A tensor whose allocation   */
+/* (when the handle is one of this library's) is shorter than buffer_sizes[i] */
+/* is skipped, as the reference does (bridge_optimizer.m:427-436).            */
+/* ------------------------------------------------------------------------ */
+
+/* bridge_optimizer.h:11-23 / .m:160-357.  momentum_buffers may be NULL or hold
+ * 0 entries: those tensors take the vanilla path.  A tensor whose weight or
+ * gradient handle is 0 is skipped (.m:199-202).  -10: HIP error. */
+int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                              uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                              int num_weights, int *buffer_sizes, float learning_rate,
+                              float momentum, float weight_decay, int nesterov, int step_count);
+
+/* bridge_optimizer.h:26-40 / .m:360-641.  -4: a weight / gradient / momentum /
+ * variance handle is 0 (nothing is updated); -6: HIP error. */
+int execute_adam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                               uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                               uintptr_t *variance_buffers, int num_weights, int *buffer_sizes,
+                               float learning_rate, float beta1, float beta2, float epsilon,
+                               float weight_decay, int step_count);
+
+/* bridge_optimizer.h:58-73 / .m:645-688.  The reference's body is a stub that
+ * validates its handles and updates nothing (and optimizer/adam.go:191-227
+ * never calls it).  Here: -1 device 0, -15 command_pool 0, otherwise the same
+ * step as execute_adam_step_mpsgraph. */
+int execute_adam_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                      uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                                      uintptr_t *variance_buffers, int num_weights,
+                                      int *buffer_sizes, float learning_rate, float beta1,
+                                      float beta2, float epsilon, float weight_decay,
+                                      int step_count, uintptr_t command_pool);
+
+/* bridge_optimizer.h:76-92 / .m:691-951.  -4: weight / gradient / squared-avg
+ * handle 0; -5: momentum > 0 with a 0 momentum handle; -6: centered with a 0
+ * gradient-average handle; -8: HIP error.  The momentum and gradient-average
+ * states ARE written back (the reference omits them from its feeds and
+ * targets, .m:909-915, so its momentum / centered variants cannot run). */
+int execute_rmsprop_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                  uintptr_t *gradient_buffers,
+                                  uintptr_t *squared_grad_avg_buffers,
+                                  uintptr_t *momentum_buffers, uintptr_t *gradient_avg_buffers,
+                                  int num_weights, int *buffer_sizes, float learning_rate,
+                                  float alpha, float epsilon, float weight_decay, float momentum,
+                                  bool centered, int step_count);
+
+/* bridge_optimizer.h:97-120 / .m:1421-1674.  A tensor with a 0 handle is
+ * skipped.  -8: HIP error.  _pooled ignores command_pool (0 or not). */
+int execute_adagrad_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                  uintptr_t *gradient_buffers,
+                                  uintptr_t *squared_grad_avg_buffers, int num_weights,
+                                  int *buffer_sizes, float learning_rate, float epsilon,
+                                  float weight_decay);
+int execute_adagrad_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                         uintptr_t *gradient_buffers,
+                                         uintptr_t *squared_grad_avg_buffers, int num_weights,
+                                         int *buffer_sizes, float learning_rate, float epsilon,
+                                         float weight_decay, uintptr_t command_pool);
+
+/* bridge_optimizer.h:125-150 / .m:1708-2019.  As AdaGrad. */
+int execute_adadelta_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                   uintptr_t *gradient_buffers,
+                                   uintptr_t *squared_grad_avg_buffers,
+                                   uintptr_t *squared_update_avg_buffers, int num_weights,
+                                   int *buffer_sizes, float rho, float epsilon,
+                                   float weight_decay);
+int execute_adadelta_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                          uintptr_t *gradient_buffers,
+                                          uintptr_t *squared_grad_avg_buffers,
+                                          uintptr_t *squared_update_avg_buffers,
+                                          int num_weights, int *buffer_sizes, float rho,
+                                          float epsilon, float weight_decay,
+                                          uintptr_t command_pool);
+
+/* bridge_optimizer.h:207-221 / .m:2023-2280.  -4: a handle is 0; -6: HIP error. */
+int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
+                                uintptr_t *variance_buffers, int num_weights, int *buffer_sizes,
+                                float learning_rate, float beta1, float beta2, float epsilon,
+                                float weight_decay, int step_count);
+
+/* ------------------------------------------------------------------------ */
+/* Additions (no counterpart in the reference's C ABI).                       */
+/* ------------------------------------------------------------------------ */
+
+/* Blocks until everything enqueued on the device's stream has finished.
+ * -1: device 0; -3: no GPU; -10: HIP error (a kernel fault surfaces here). */
+int gm_synchronize(uintptr_t device);
+
+/* Message of the most recent failure on the calling thread ("" if none). */
+const char *gm_last_error(void);
+
+/* Allocation length in bytes of one of this library's buffers; 0 if unknown. */
+size_t gm_buffer_length(uintptr_t buffer);
+
+/* Host-side step scalars, exactly as the update entry points compute them
+ * (bridge_optimizer.m:398-399, :2066). */
+void  gm_bias_corrections(float beta1, float beta2, int step_count, float *bc1, float *bc2);
+float gm_nadam_mu_next(float beta1, int step_count);
+
+/* Dynamic loss-scale state for the mixed-precision Adam step, resident on the
+ * device.  Defaults in the reference's trainer config: 65536, 2.0, 0.5, 2000
+ * (training/model_trainer.go:258-270).  The reference itself never unscales,
+ * checks or rescales (it only stores those constants); this step is the
+ * algorithm its tutorial describes (docs/tutorials/mixed-precision.md:610-629). */
+uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_factor,
+                              float backoff_factor, int growth_interval);
+void gm_amp_state_destroy(uintptr_t amp_state);
+/* Reads / overwrites scale and the clean-step counter (checkpointing). */
+int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker);
+int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker);
+
+/* One mixed-precision Adam step over the whole tensor list.
+ *   gradient16_buffers: fp16 gradients of the SCALED loss (read only)
+ *   weight/momentum/variance_buffers: fp32 master state, updated in place
+ *   weight16_buffers: fp16 copy of the updated weights (entries may be 0 or
+ *                     the array NULL: no copy is emitted for those tensors)
+ *   buffer_sizes: bytes of the fp32 weight tensor (numel = size / 4)
+ *   step_count: the bias-correction step to use IF the step is applied
+ * If any gradient element of any tensor is +-inf or NaN the step is skipped:
+ * no buffer is written, scale *= backoff, clean-step counter = 0, *skipped = 1.
+ * Otherwise g = float(g16) * (1.0f / scale), the Adam rule of
+ * execute_adam_step_mpsgraph, w16 = half(w'), counter++, and scale *= growth
+ * when the counter reaches growth_interval; *skipped = 0.
+ * The call synchronises the stream (it reports *skipped).  scale_out /
+ * growth_tracker_out (may be NULL) receive the state after the step.
+ * -1 device 0; -3 no GPU; -4 a required handle is 0; -6 HIP error; -16 amp_state 0. */
+int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
+                          uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                          uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                          int num_weights, int *buffer_sizes, float learning_rate, float beta1,
+                          float beta2, float epsilon, float weight_decay, int step_count,
+                          uintptr_t amp_state, int *skipped, float *scale_out,
+                          int *growth_tracker_out);
+
+/* Measurement helpers used by the benchmark and the profiles. */
+
+/* Records a start / stop event pair on the device's stream; gm_timer_stop
+ * synchronises and returns the elapsed milliseconds between them (< 0 on error). */
+int   gm_timer_start(uintptr_t device);
+float gm_timer_stop(uintptr_t device);
+/* Fills a buffer with counter-based pseudo-random normals N(mean, std) (fp32)
+ * or half(N(mean, std) * scale) (fp16), reproducible from (seed, element index). */
+int gm_fill_normal_f32(uintptr_t device, uintptr_t buffer, size_t num_elements, uint64_t seed,
+                       float mean, float std);
+int gm_fill_normal_f16(uintptr_t device, uintptr_t buffer, size_t num_elements, uint64_t seed,
+                       float mean, float std, float scale);
+/* Plain 16-byte-per-lane copy kernel: the measured HBM ceiling the update
+ * kernels are compared with, and the known-size launch that calibrates the
+ * profiler's FETCH_SIZE / WRITE_SIZE counters. */
+int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, size_t bytes);
+/* Launch-shape overrides for sweeps: elements per workgroup-chunk (multiple of
+ * 1024, 0 = default) and non-temporal memory hints on/off (-1 = default). */
+int gm_set_tuning(int chunk_elements, int nontemporal);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,163 @@
+"""GPU parity: libgometal_hip.so (through the C ABI) against the CPU oracle and the golden
+vectors.  fp32 rules are required to be BIT-IDENTICAL to the oracle (the stated tolerance is
+<= 2 ulp after 10 steps; the kernels evaluate the same IEEE operations in the same order, so
+the tests hold them to 0 ulp and fail on any difference)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from harness import GpuRun, OracleRun, compare_snapshots, gpu_device
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "optimizer_kat.json")) as f:
+    KAT = json.load(f)
+
+NTHREADS = min(16, os.cpu_count() or 1)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = gpu_device()
+    if d is None:
+        pytest.fail("libgometal_hip.so is missing or no GPU is usable: GPU tests cannot run")
+    return d
+
+
+def f32(bits):
+    return np.array(bits, dtype=np.uint32).view(np.float32).copy()
+
+
+@pytest.mark.parametrize("case", KAT["cases"], ids=[c["name"] for c in KAT["cases"]])
+def test_golden_vectors(dev, case):
+    """Known-answer vectors (exact-rational evaluator), incl. the reference's own test inputs."""
+    run = GpuRun(dev, case["rule"], case["hyper"], [f32(case["w0"])])
+    run.step_count = case["first_step"] - 1
+    try:
+        for k, gbits in enumerate(case["grads"]):
+            run.step([f32(gbits)])
+            got = run.snapshot()
+            for key in got:
+                assert got[key][0].view(np.uint32).tolist() == case["expect"][k][key], (case["name"], k, key)
+    finally:
+        run.close()
+
+
+def run_both(dev, rule, hyper, weights, grad_fn, steps, check_every=1, nthreads=NTHREADS):
+    gpu = GpuRun(dev, rule, hyper, weights)
+    cpu = OracleRun(rule, hyper, weights, nthreads=nthreads)
+    try:
+        for k in range(steps):
+            grads = grad_fn(k)
+            gpu.step(grads)
+            cpu.step(grads)
+            if (k + 1) % check_every == 0 or k == steps - 1:
+                compare_snapshots(gpu.snapshot(), cpu.snapshot(), max_ulp=0, context=f"{rule} step {k + 1}")
+    finally:
+        gpu.close()
+
+
+def test_config1_adam_flat_1m(dev):
+    """One flat tensor of 1,048,576 params, N(0, 0.02); grads N(0, 1e-2); 10 steps, p/m/v after every step."""
+    rng = np.random.default_rng(0x6D657461 + 1)
+    n = 1 << 20
+    w = [rng.normal(0, 0.02, n).astype(np.float32)]
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)
+    run_both(dev, "adam", hyper, w, lambda k: [rng.normal(0, 1e-2, n).astype(np.float32)], steps=10)
+
+
+CNN_SHAPES = [
+    (32, 3, 3, 3), (32,), (64, 32, 3, 3), (64,), (128, 64, 3, 3), (128,),   # conv weights + biases
+    (32,), (32,), (64,), (64,), (128,), (128,),                           # BatchNorm gamma / beta
+    (8192, 128), (128,), (128, 10), (10,),                                # dense
+]
+
+
+@pytest.mark.parametrize("rule,hyper", [
+    ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=0.0, nesterov=False)),
+    ("adam", dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)),
+])
+def test_config2_cnn_parameter_list(dev, rule, hyper):
+    """16 tensors / 1,143,690 params, weights N(0, 0.02), grads N(0, 1e-3), 100 steps."""
+    rng = np.random.default_rng(0x6D657461 + 2)
+    sizes = [int(np.prod(s)) for s in CNN_SHAPES]
+    assert sum(sizes) == 1143690
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
+             steps=100, check_every=10)
+
+
+def ragged_sizes(count=160, total=25_000_000, lo=64, hi=4 * 1024 * 1024, seed=0x6D657461 + 3):
+    """160 sizes, log-uniform in [64, 4M], rescaled so they sum to `total`."""
+    rng = np.random.default_rng(seed)
+    raw = np.exp(rng.uniform(np.log(lo), np.log(hi), count))
+    sizes = np.maximum(lo, np.floor(raw * (total / raw.sum()))).astype(np.int64)
+    sizes = np.minimum(sizes, hi)
+    # put the rounding remainder on the largest tensor that has room
+    diff = total - int(sizes.sum())
+    order = np.argsort(-sizes)
+    for idx in order:
+        room = hi - sizes[idx] if diff > 0 else sizes[idx] - lo
+        take = int(np.sign(diff) * min(abs(diff), room))
+        sizes[idx] += take
+        diff -= take
+        if diff == 0:
+            break
+    assert int(sizes.sum()) == total and sizes.min() >= lo and sizes.max() <= hi
+    return [int(s) for s in sizes]
+
+
+CONFIG3 = [
+    ("rmsprop", dict(lr=0.01, alpha=0.99, eps=1e-8, weight_decay=0.0, momentum=0.0, centered=False)),
+    ("adagrad", dict(lr=0.01, eps=1e-10, weight_decay=0.0)),
+    ("adadelta", dict(rho=0.9, eps=1e-6, weight_decay=0.0)),
+    ("nadam", dict(lr=0.002, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)),
+]
+
+
+@pytest.fixture(scope="module")
+def config3_data():
+    """25M params in 160 ragged tensors; a pool of 4 heavy-tailed gradient sets that the
+    50 steps cycle through (N(0, 1e-3), a seeded 1% of elements x100)."""
+    sizes = ragged_sizes()
+    rng = np.random.default_rng(0x6D657461 + 30)
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    pool = []
+    for _ in range(4):
+        gs = []
+        for n in sizes:
+            g = rng.normal(0, 1e-3, n).astype(np.float32)
+            g[rng.random(n) < 0.01] *= np.float32(100.0)
+            gs.append(g)
+        pool.append(gs)
+    return sizes, w, pool
+
+
+@pytest.mark.parametrize("rule,hyper", CONFIG3, ids=[c[0] for c in CONFIG3])
+def test_config3_ragged_25m(dev, config3_data, rule, hyper):
+    sizes, w, pool = config3_data
+    run_both(dev, rule, hyper, w, lambda k: pool[k % len(pool)], steps=50, check_every=25)
+
+
+@pytest.mark.parametrize("rule,hyper", [
+    ("rmsprop", dict(lr=0.01, alpha=0.99, eps=1e-8, weight_decay=1e-4, momentum=0.9, centered=True)),
+    ("rmsprop", dict(lr=0.01, alpha=0.99, eps=1e-8, weight_decay=0.0, momentum=0.9, centered=False)),
+    ("rmsprop", dict(lr=0.01, alpha=0.99, eps=1e-8, weight_decay=0.0, momentum=0.0, centered=True)),
+    ("sgd", dict(lr=0.01, momentum=0.0, weight_decay=5e-4, nesterov=False)),
+    ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=5e-4, nesterov=True)),
+    ("adagrad", dict(lr=0.01, eps=1e-10, weight_decay=1e-3)),
+    ("adadelta", dict(rho=0.95, eps=1e-6, weight_decay=1e-3)),
+    ("nadam", dict(lr=0.002, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)),
+    ("adam", dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)),
+])
+def test_variants_and_ragged_edges(dev, rule, hyper):
+    """Every rule variant over sizes that exercise the vector body, the scalar tail, one-element
+    tensors, an empty tensor and chunk boundaries (chunk = 65536 elements)."""
+    rng = np.random.default_rng(99)
+    sizes = [1, 2, 3, 4, 5, 0, 63, 64, 65, 1023, 1024, 1025, 4095, 4097, 65535, 65536, 65537, 131072 + 7, 300001]
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
+             steps=6, check_every=3, nthreads=1)
