@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the optimizer-step hot path on one MI355X.
+
+A "step" is one optimizer step over the whole synthetic parameter list of the chosen
+workload, with weights, gradients and state already resident in HBM.  The default workload
+is the headline configuration: Adam with weight decay 1e-4 over 1,012,301,824 fp32
+parameters in 400 tensors shaped like transformer blocks.
+
+Prints ONE JSON line: params updated per second (whole job), ms per step, the roofline of
+the dominant kernel (algorithmic bytes per launch / launch duration measured with HIP
+events on the library's own stream, against MI355X's 8 TB/s HBM peak), the same figures for
+the mixed-precision (fp16 gradient) Adam step, and the CPU oracle timed on this host's cores
+on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+# algorithmic bytes per parameter per step: every stream read once and / or written once
+BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelta": 28, "nadam": 28,
+                   "adam_amp": 28}
+
+
+from workloads import amp_125m_sizes, cnn_sizes, ragged_sizes, transformer_block_sizes  # noqa: E402
+
+WORKLOADS = {
+    # name: (description, sizes(), rule, hyper, gradient std)
+    "c1": ("config1: Adam, one flat tensor of 1,048,576 params", lambda: [1 << 20], "adam",
+           dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0), 1e-2),
+    "c2-sgd": ("config2: SGD-momentum over the 16-tensor CNN list (1,143,690 params)", cnn_sizes, "sgd",
+               dict(lr=0.01, momentum=0.9, weight_decay=0.0, nesterov=False), 1e-3),
+    "c2-adam": ("config2: Adam over the 16-tensor CNN list (1,143,690 params)", cnn_sizes, "adam",
+                dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0), 1e-3),
+    "c3-rmsprop": ("config3: RMSprop, 25M params in 160 ragged tensors", ragged_sizes, "rmsprop",
+                   dict(lr=0.01, alpha=0.99, eps=1e-8, weight_decay=0.0, momentum=0.0, centered=False), 1e-3),
+    "c3-adagrad": ("config3: AdaGrad, 25M params in 160 ragged tensors", ragged_sizes, "adagrad",
+                   dict(lr=0.01, eps=1e-10, weight_decay=0.0), 1e-3),
+    "c3-adadelta": ("config3: AdaDelta, 25M params in 160 ragged tensors", ragged_sizes, "adadelta",
+                    dict(rho=0.9, eps=1e-6, weight_decay=0.0), 1e-3),
+    "c3-nadam": ("config3: NAdam, 25M params in 160 ragged tensors", ragged_sizes, "nadam",
+                 dict(lr=0.002, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0), 1e-3),
+    "c4": ("config4: mixed-precision Adam, 125M params in 60 tensors", amp_125m_sizes, "adam",
+           dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0), 1e-4),
+    "c5": ("config5: Adam + weight decay 1e-4, 1,012,301,824 params in 400 transformer-block tensors",
+           transformer_block_sizes, "adam",
+           dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4), 1e-4),
+}
+
+
+def time_steps(dev, launch, steps, warmup):
+    """W untimed steps, then exactly K steps bracketed by a device synchronisation on both
+    sides.  Returns (wall ms per step, HIP-event ms per launch)."""
+    for _ in range(warmup):
+        launch()
+    dev.synchronize()
+    t0 = time.perf_counter()
+    dev.lib.gm_timer_start(dev.handle)
+    for _ in range(steps):
+        launch()
+    event_ms = dev.lib.gm_timer_stop(dev.handle)     # records the stop event and waits for it
+    dev.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms / steps, event_ms / steps
+
+
+def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_seconds=12.0):
+    """The CPU oracle (a C port of the reference's update equations, OpenMP over elements) on
+    this host, on the leading tensors of the same workload up to ~budget_params, for about
+    target_seconds of CPU work."""
+    from oracle_lib import oracle
+    from harness import OracleRun
+    oracle()
+    threads = min(16, os.cpu_count() or 1)
+    chosen, total = [], 0
+    for n in sizes:
+        if chosen and total + n > budget_params:
+            break
+        chosen.append(n)
+        total += n
+    rng = np.random.default_rng(1)
+    w = [rng.standard_normal(n, dtype=np.float32) * np.float32(0.02) for n in chosen]
+    g = [rng.standard_normal(n, dtype=np.float32) * np.float32(grad_std) for n in chosen]
+    run = OracleRun(rule, hyper, w, nthreads=threads)
+    run.step(g)                                   # warm-up (page faults, thread pool)
+    t0 = time.perf_counter()
+    run.step(g)
+    one = max(time.perf_counter() - t0, 1e-4)
+    steps = int(min(2000, max(3, target_seconds / one)))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run.step(g)
+    dt = time.perf_counter() - t0
+    return {"value": total * steps / dt, "unit": "params/s", "cores": threads, "kind": "port",
+            "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} steps in "
+                      f"{dt:.1f} s, oracle/oracle.c with OpenMP on {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-amp", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the optimizer step shards without communication, and this "
+                 "build runs and reports a single MI355X (--gpus 1).")
+
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    dev = pkg.Device()                 # raises if the library is not built or no GPU is visible
+    lib, D = dev.lib, dev.handle
+
+    desc, sizes_fn, rule, hyper, grad_std = WORKLOADS[args.workload]
+    sizes = sizes_fn()
+    n = len(sizes)
+    params = sum(sizes)
+    nstate = {"sgd": 1, "adam": 2, "rmsprop": 1, "adagrad": 1, "adadelta": 2, "nadam": 2}[rule]
+
+    # ---- synthetic data, generated on the device ----
+    w = [dev.alloc(4 * s) for s in sizes]
+    g = [dev.alloc(4 * s) for s in sizes]
+    states = [[dev.alloc(4 * s, zero=True) for s in sizes] for _ in range(nstate)]
+    for k, s in enumerate(sizes):
+        lib.gm_fill_normal_f32(D, w[k], s, 0x6D657461 + k, 0.0, 0.02)
+        lib.gm_fill_normal_f32(D, g[k], s, 0x12345 + k, 0.0, grad_std)
+    dev.synchronize()
+    cw, cg = pkg.handle_array(w), pkg.handle_array(g)
+    cs = [pkg.handle_array(s) for s in states]
+    bs = pkg.int_array([4 * s for s in sizes])
+    counter = {"t": 0}
+
+    def launch_fp32():
+        counter["t"] += 1
+        t = counter["t"]
+        h = hyper
+        if rule == "adam":
+            rc = lib.execute_adam_step_mpsgraph(D, cw, cg, cs[0], cs[1], n, bs, h["lr"], h["beta1"], h["beta2"],
+                                                h["eps"], h["weight_decay"], t)
+        elif rule == "nadam":
+            rc = lib.execute_nadam_step_mpsgraph(D, cw, cg, cs[0], cs[1], n, bs, h["lr"], h["beta1"], h["beta2"],
+                                                 h["eps"], h["weight_decay"], t)
+        elif rule == "sgd":
+            rc = lib.execute_sgd_step_mpsgraph(D, cw, cg, cs[0], n, bs, h["lr"], h["momentum"],
+                                               h["weight_decay"], int(h["nesterov"]), t)
+        elif rule == "rmsprop":
+            rc = lib.execute_rmsprop_step_mpsgraph(D, cw, cg, cs[0], None, None, n, bs, h["lr"], h["alpha"],
+                                                   h["eps"], h["weight_decay"], h["momentum"], False, t)
+        elif rule == "adagrad":
+            rc = lib.execute_adagrad_step_mpsgraph(D, cw, cg, cs[0], n, bs, h["lr"], h["eps"], h["weight_decay"])
+        else:
+            rc = lib.execute_adadelta_step_mpsgraph(D, cw, cg, cs[0], cs[1], n, bs, h["rho"], h["eps"],
+                                                    h["weight_decay"])
+        if rc != 0:
+            raise RuntimeError(f"{rule} step failed rc={rc}: {lib.gm_last_error().decode()}")
+
+    wall_ms, event_ms = time_steps(dev, launch_fp32, args.steps, args.warmup)
+    bpp = BYTES_PER_PARAM[rule]
+    achieved = params * bpp / (event_ms * 1e-3) / 1e9
+
+    # measured ceiling: plain 16-byte copy kernel, same box, same run
+    probe_bytes = min(1 << 30, max(1 << 24, (4 * max(sizes)) // 16 * 16))
+    src, dst = dev.alloc(probe_bytes), dev.alloc(probe_bytes)
+    _, copy_ms = time_steps(dev, lambda: lib.gm_copy_probe(D, dst, src, probe_bytes), 10, 3)
+    copy_gbs = 2 * probe_bytes / (copy_ms * 1e-3) / 1e9
+    dev.free(src)
+    dev.free(dst)
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(f"{args.workload}:{rule}")
+
+    result = {
+        "metric": "params updated/sec (Adam fp32 multi-tensor step) + achieved HBM GB/s (% of peak)"
+                  if rule == "adam" else f"params updated/sec ({rule} multi-tensor step) + achieved HBM GB/s",
+        "value": params / (wall_ms * 1e-3),
+        "unit": "params/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": desc, "tensors": n, "params": params, "rule": rule, "hyper": hyper},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": f"multi_tensor_update_kernel<{rule}>", "bytes_per_param": bpp,
+                     "kernel_ms": event_ms, "copy_kernel_gbs": copy_gbs,
+                     "frac_of_copy_kernel": achieved / copy_gbs},
+    }
+
+    # ---- mixed-precision Adam on the same list (fp16 gradients, fp16 weight copy) ----
+    if rule == "adam" and not args.no_amp:
+        g16 = [dev.alloc(2 * s) for s in sizes]
+        w16 = [dev.alloc(2 * s) for s in sizes]
+        for k, s in enumerate(sizes):
+            lib.gm_fill_normal_f16(D, g16[k], s, 0x777 + k, 0.0, grad_std, 65536.0)
+        dev.synchronize()
+        cg16, cw16 = pkg.handle_array(g16), pkg.handle_array(w16)
+        amp = lib.gm_amp_state_create(D, 65536.0, 2.0, 0.5, 2000)
+        skipped, scale, tracker = ctypes.c_int(), ctypes.c_float(), ctypes.c_int()
+        amp_t = {"t": 0, "skipped": 0}
+
+        def launch_amp():
+            rc = lib.execute_adam_amp_step(D, cw, cg16, cs[0], cs[1], cw16, n, bs, hyper["lr"], hyper["beta1"],
+                                           hyper["beta2"], hyper["eps"], hyper["weight_decay"], amp_t["t"] + 1,
+                                           amp, ctypes.byref(skipped), ctypes.byref(scale), ctypes.byref(tracker))
+            if rc != 0:
+                raise RuntimeError(f"mixed-precision step failed rc={rc}: {lib.gm_last_error().decode()}")
+            if skipped.value:
+                amp_t["skipped"] += 1
+            else:
+                amp_t["t"] += 1
+
+        amp_wall, amp_event = time_steps(dev, launch_amp, args.steps, args.warmup)
+        amp_achieved = params * BYTES_PER_PARAM["adam_amp"] / (amp_wall * 1e-3) / 1e9
+        result["amp"] = {
+            "value": params / (amp_wall * 1e-3), "unit": "params/s", "ms_per_step": amp_wall,
+            "dtype": "f32 master state, f16 gradients and weight copy", "skipped_steps": amp_t["skipped"],
+            "roofline": {"bound": "hbm", "achieved": amp_achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": amp_achieved / HBM_PEAK_GBS, "bytes_per_param": 28,
+                         "bytes_per_param_moved": 30,
+                         "note": "step time covers the overflow-check launch, the update launch and the "
+                                 "read-back of the skip flag; each step is synchronous"},
+        }
+        lib.gm_amp_state_destroy(amp)
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(sizes, rule, hyper, grad_std)
+    else:
+        result["cpu_baseline"] = None
+
+    dev.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

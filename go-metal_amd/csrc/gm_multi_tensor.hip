@@ -170,18 +170,26 @@ MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req)
 }
 
 // --------------------------------------------------------------- kernels ----
+// Tensor addresses reach the kernels through tables in memory, so the compiler
+// only knows them as generic pointers and would emit flat_* instructions.  They
+// are always HBM addresses: casting to the global address space yields
+// global_load / global_store (one wait counter, no aperture check).
+#define GM_GLOBAL __attribute__((address_space(1)))
+
 template <bool NT, class T>
 __device__ inline T stream_load(const T *p)
 {
-    if (NT) return __builtin_nontemporal_load(p);
-    return *p;
+    const GM_GLOBAL T *gp = (const GM_GLOBAL T *)p;
+    if (NT) return __builtin_nontemporal_load(gp);
+    return *gp;
 }
 
 template <bool NT, class T>
 __device__ inline void stream_store(T v, T *p)
 {
-    if (NT) __builtin_nontemporal_store(v, p);
-    else *p = v;
+    GM_GLOBAL T *gp = (GM_GLOBAL T *)p;
+    if (NT) __builtin_nontemporal_store(v, gp);
+    else *gp = v;
 }
 
 // Applies Rule to `count` elements starting at element `offset` of a tensor.
@@ -262,16 +270,16 @@ __device__ inline void process_chunk(const TensorRec &rec, uint64_t offset, uint
     }
     // scalar path: the < 4 element tail, or the whole chunk when a stream is misaligned
     for (uint32_t i = done + threadIdx.x; i < count; i += kBlock) {
-        float wv = w[i];
-        float gv = AMP ? (float)g16[i] * inv_scale : g32[i];
+        float wv = stream_load<false>(w + i);
+        float gv = AMP ? (float)stream_load<false>(g16 + i) * inv_scale : stream_load<false>(g32 + i);
         float sv[NSA];
 #pragma unroll
-        for (int k = 0; k < NS; k++) sv[k] = st[k][i];
+        for (int k = 0; k < NS; k++) sv[k] = stream_load<false>(st[k] + i);
         Rule::apply(wv, gv, sv, prm);
-        w[i] = wv;
+        stream_store<false>(wv, w + i);
 #pragma unroll
-        for (int k = 0; k < NS; k++) st[k][i] = sv[k];
-        if (AMP && w16) w16[i] = (_Float16)wv;
+        for (int k = 0; k < NS; k++) stream_store<false>(sv[k], st[k] + i);
+        if (AMP && w16) stream_store<false>((_Float16)wv, w16 + i);
     }
 }
 
@@ -306,7 +314,7 @@ struct AmpDeviceState {
     float scale;
     int growth_tracker;
     int found_inf;          // set by the check kernel, consumed and cleared by the update kernel
-    unsigned int ticket;    // workgroups of the update kernel that have finished
+    unsigned int reserved;
     int last_skipped;
     float growth_factor;
     float backoff_factor;
@@ -363,46 +371,43 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, const TensorRec *__r
 }
 
 // Phase B: the Adam update on unscaled gradients, skipped as a whole when the
-// flag is set; the last workgroup to finish advances the loss-scale state.
+// flag is set.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
-                       uint32_t num_chunks, StepParams prm, AmpDeviceState *state)
+                       StepParams prm, const AmpDeviceState *__restrict__ state)
 {
-    const int found = *reinterpret_cast<volatile int *>(&state->found_inf);
-    const float scale = *reinterpret_cast<volatile float *>(&state->scale);
-    if (!found && blockIdx.x < num_chunks) {
-        const float inv_scale = 1.0f / scale;
-        const Chunk ch = chunks[blockIdx.x];
-        const TensorRec rec = recs[ch.tensor];
-        process_chunk<AdamRule, NT, true>(rec, ch.offset, ch.count, prm, inv_scale);
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __threadfence();
-        const unsigned int t = atomicAdd(&state->ticket, 1u);
-        if (t == gridDim.x - 1) {
-            // Every other workgroup has read the flag and the scale and finished.
-            float s = scale;
-            int tracker = state->growth_tracker;
-            if (found) {
-                s = s * state->backoff_factor;
-                tracker = 0;
-            } else {
-                tracker += 1;
-                if (tracker == state->growth_interval) {
-                    s = s * state->growth_factor;
-                    tracker = 0;
-                }
-            }
-            state->scale = s;
-            state->growth_tracker = tracker;
-            state->last_skipped = found ? 1 : 0;
-            state->found_inf = 0;
-            state->ticket = 0;
-            __threadfence();
+    if (state->found_inf) return;
+    const float inv_scale = 1.0f / state->scale;
+    const Chunk ch = chunks[blockIdx.x];
+    const TensorRec rec = recs[ch.tensor];
+    process_chunk<AdamRule, NT, true>(rec, ch.offset, ch.count, prm, inv_scale);
+}
+
+// Epilogue (one lane, same stream, after phase B has drained): advances the
+// loss-scale state machine and re-arms the flag.  A separate launch rather
+// than a last-workgroup ticket: a single counter bumped by every workgroup of
+// a 250k-workgroup grid serialises in the memory-side atomic unit.
+__global__ void amp_finalize_kernel(AmpDeviceState *state)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const int found = state->found_inf;
+    float s = state->scale;
+    int tracker = state->growth_tracker;
+    if (found) {
+        s = s * state->backoff_factor;
+        tracker = 0;
+    } else {
+        tracker += 1;
+        if (tracker == state->growth_interval) {
+            s = s * state->growth_factor;
+            tracker = 0;
         }
     }
+    state->scale = s;
+    state->growth_tracker = tracker;
+    state->last_skipped = found ? 1 : 0;
+    state->found_inf = 0;
 }
 
 // ----------------------------------------------------------- host helpers ----
@@ -859,21 +864,21 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
     gm_bias_corrections(beta1, beta2, step_count, &p.bc1, &p.bc2);
 
     const uint32_t chunks = l.plan->num_chunks;
-    const uint32_t grid = chunks > 0 ? chunks : 1;
     hipStream_t st = l.ctx->stream;
-    if (current_nontemporal()) {
-        if (chunks > 0)
+    if (chunks > 0) {
+        if (current_nontemporal()) {
             amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs,
                                                                       amp->d_state);
-        amp_adam_update_kernel<true><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, chunks,
-                                                             p, amp->d_state);
-    } else {
-        if (chunks > 0)
+            amp_adam_update_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, p,
+                                                                   amp->d_state);
+        } else {
             amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs,
                                                                        amp->d_state);
-        amp_adam_update_kernel<false><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, chunks,
-                                                              p, amp->d_state);
+            amp_adam_update_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, p,
+                                                                    amp->d_state);
+        }
     }
+    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state);
     if (!hip_ok(hipGetLastError(), "mixed-precision kernel launch")) return -6;
     if (!amp_download(amp)) return -6;
     if (skipped) *skipped = amp->h_pinned->last_skipped;

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from harness import GpuRun, OracleRun, compare_snapshots, gpu_device
+from workloads import cnn_sizes, ragged_sizes
 
 pytestmark = pytest.mark.gpu
 
@@ -69,13 +70,6 @@ def test_config1_adam_flat_1m(dev):
     run_both(dev, "adam", hyper, w, lambda k: [rng.normal(0, 1e-2, n).astype(np.float32)], steps=10)
 
 
-CNN_SHAPES = [
-    (32, 3, 3, 3), (32,), (64, 32, 3, 3), (64,), (128, 64, 3, 3), (128,),   # conv weights + biases
-    (32,), (32,), (64,), (64,), (128,), (128,),                           # BatchNorm gamma / beta
-    (8192, 128), (128,), (128, 10), (10,),                                # dense
-]
-
-
 @pytest.mark.parametrize("rule,hyper", [
     ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=0.0, nesterov=False)),
     ("adam", dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)),
@@ -83,31 +77,10 @@ CNN_SHAPES = [
 def test_config2_cnn_parameter_list(dev, rule, hyper):
     """16 tensors / 1,143,690 params, weights N(0, 0.02), grads N(0, 1e-3), 100 steps."""
     rng = np.random.default_rng(0x6D657461 + 2)
-    sizes = [int(np.prod(s)) for s in CNN_SHAPES]
-    assert sum(sizes) == 1143690
+    sizes = cnn_sizes()
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
     run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
              steps=100, check_every=10)
-
-
-def ragged_sizes(count=160, total=25_000_000, lo=64, hi=4 * 1024 * 1024, seed=0x6D657461 + 3):
-    """160 sizes, log-uniform in [64, 4M], rescaled so they sum to `total`."""
-    rng = np.random.default_rng(seed)
-    raw = np.exp(rng.uniform(np.log(lo), np.log(hi), count))
-    sizes = np.maximum(lo, np.floor(raw * (total / raw.sum()))).astype(np.int64)
-    sizes = np.minimum(sizes, hi)
-    # put the rounding remainder on the largest tensor that has room
-    diff = total - int(sizes.sum())
-    order = np.argsort(-sizes)
-    for idx in order:
-        room = hi - sizes[idx] if diff > 0 else sizes[idx] - lo
-        take = int(np.sign(diff) * min(abs(diff), room))
-        sizes[idx] += take
-        diff -= take
-        if diff == 0:
-            break
-    assert int(sizes.sum()) == total and sizes.min() >= lo and sizes.max() <= hi
-    return [int(s) for s in sizes]
 
 
 CONFIG3 = [
@@ -155,9 +128,10 @@ def test_config3_ragged_25m(dev, config3_data, rule, hyper):
 ])
 def test_variants_and_ragged_edges(dev, rule, hyper):
     """Every rule variant over sizes that exercise the vector body, the scalar tail, one-element
-    tensors, an empty tensor and chunk boundaries (chunk = 65536 elements)."""
+    tensors, an empty tensor and chunk boundaries (a workgroup chunk is 4096 elements)."""
     rng = np.random.default_rng(99)
-    sizes = [1, 2, 3, 4, 5, 0, 63, 64, 65, 1023, 1024, 1025, 4095, 4097, 65535, 65536, 65537, 131072 + 7, 300001]
+    sizes = [1, 2, 3, 4, 5, 0, 63, 64, 65, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8193, 65535, 65537, 131072 + 7,
+             300001]
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
     run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
              steps=6, check_every=3, nthreads=1)
