@@ -64,7 +64,7 @@ ABI = {
     "gm_fill_normal_f32": (i, [u, u, ctypes.c_size_t, ctypes.c_uint64, f, f]),
     "gm_fill_normal_f16": (i, [u, u, ctypes.c_size_t, ctypes.c_uint64, f, f, f]),
     "gm_copy_probe": (i, [u, u, u, ctypes.c_size_t]),
-    "gm_set_tuning": (i, [i, i]),
+    "gm_set_tuning": (i, [i, i, i]),
 }
 
 _LIB = None

@@ -2,12 +2,21 @@
 // the execute_*_step entry points of the C ABI (the HIP counterpart of
 // cgo_bridge/bridge_optimizer.m).
 //
-// One launch per step.  Workgroup b walks chunk b of the device-side chunk
-// table: 256 lanes, each lane moving 16-byte vectors (global_load_dwordx4 /
-// global_store_dwordx4), UNROLL vectors of every stream in flight before the
-// first use, every state read once and written once, fp32 throughout.  The
-// path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS staging and
-// no MFMA, only enough independent loads per lane to cover HBM latency.
+// One launch per step.  The parameter list is cut into chunks of
+// chunk_elements (default 16384) and each chunk into slices of 256 * VEC
+// elements; workgroup b handles slice (b mod slices_per_chunk) of chunk
+// (b div slices_per_chunk), one VEC-wide group per lane: load every stream
+// once, apply the rule in registers, store every state once, exit.
+//
+// VEC = 1 (one fp32 per lane, global_load_dword) is the default: measured on
+// MI355X it sustains about 85 % of peak HBM bandwidth on the 4-read / 3-write
+// Adam stream, against about 80 % for 8-byte and 72-77 % for 16-byte lanes
+// (global_load_dwordx4), whatever the unrolling or workgroup size.  Short
+// single-pass waves keep reads and writes finely interleaved at the memory
+// controllers; wide, unrolled lanes issue them in bursts.  The wider
+// variants stay selectable (gm_set_tuning) so the comparison can be rerun.
+// The path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS
+// staging, no MFMA.
 #include "gm_context.hpp"
 #include "gm_plan.hpp"
 #include "gm_rules.hpp"
@@ -20,27 +29,35 @@
 
 namespace gm {
 
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
-typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 4;
-constexpr int kChunkGranule = kBlock * 4 * kUnroll;   // elements one pass of a workgroup covers
-constexpr int kDefaultChunkElements = kChunkGranule;
+constexpr int kDefaultChunkElements = 16384;
+constexpr int kDefaultVec = 1;
+constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 constexpr size_t kMaxCachedPlans = 16;
 
 static std::atomic<int> g_chunk_elements{kDefaultChunkElements};
 static std::atomic<int> g_nontemporal{1};
+static std::atomic<int> g_vec{kDefaultVec};
 
 int current_chunk_elements() { return g_chunk_elements.load(); }
 bool current_nontemporal() { return g_nontemporal.load() != 0; }
+int current_vec() { return g_vec.load(); }
+
+// log2(slices per chunk) for a chunk size and lane width; chunk_elements is a
+// power-of-two multiple of 256 * vec (gm_set_tuning enforces it).
+static uint32_t slice_shift_for(int chunk_elements, int vec)
+{
+    uint32_t slices = (uint32_t)(chunk_elements / (kBlock * vec));
+    uint32_t shift = 0;
+    while ((1u << shift) < slices) shift++;
+    return shift;
+}
 
 // ------------------------------------------------------------------ plan ----
 MultiTensorPlan::~MultiTensorPlan()
 {
-    if (d_recs) (void)hipFree(d_recs);
     if (d_chunks) (void)hipFree(d_chunks);
 }
 
@@ -79,9 +96,7 @@ static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanReque
     for (int k = 0; k < kNumSlots; k++)
         if (r.slot[k]) std::memcpy(plan->handles.data() + (size_t)k * n, r.slot[k], n * sizeof(uintptr_t));
 
-    std::vector<TensorRec> recs;
     std::vector<Chunk> chunks;
-    recs.reserve(n);
     for (size_t i = 0; i < n; i++) {
         uintptr_t h[kNumSlots];
         for (int k = 0; k < kNumSlots; k++) h[k] = plan->handles[(size_t)k * n + i];
@@ -106,27 +121,31 @@ static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanReque
 
         // 2. an allocation of ours that is shorter than the tensor: skip it
         //    (bridge_optimizer.m:427-436)
-        uint32_t flags = kRecVectorOk | kRecGrad16VectorOk;
+        uint32_t flags = kRecVec2Ok | kRecVec4Ok | kRecGrad16VectorOk;
         for (int k = 0; k < kNumSlots; k++) {
             if (h[k] == 0) continue;
             const bool half = (r.half_mask & (1u << k)) != 0;
             const size_t need = numel * (half ? 2 : 4);
             const size_t have = registry_length(h[k]);
             if (have != 0 && have < need) skip = true;
-            if (h[k] % (half ? 8 : 16) != 0) flags &= ~kRecVectorOk;
+            if (h[k] % (half ? 4 : 8) != 0) flags &= ~kRecVec2Ok;
+            if (h[k] % (half ? 8 : 16) != 0) flags &= ~kRecVec4Ok;
             if (half && k == kSlotGrad && h[k] % 16 != 0) flags &= ~kRecGrad16VectorOk;
         }
         if (skip) continue;
 
-        TensorRec rec;
-        for (int k = 0; k < kNumSlots; k++) rec.p[k] = reinterpret_cast<void *>(h[k]);
-        rec.flags = flags;
-        rec.pad = 0;
-        const uint32_t rec_index = (uint32_t)recs.size();
-        recs.push_back(rec);
         for (size_t off = 0; off < numel; off += (size_t)chunk) {
             const size_t left = numel - off;
-            chunks.push_back(Chunk{rec_index, (uint32_t)(left < (size_t)chunk ? left : (size_t)chunk), off});
+            Chunk c{};
+            for (int k = 0; k < kNumSlots; k++) {
+                if (h[k] == 0) continue;
+                const size_t elem = (r.half_mask & (1u << k)) ? 2 : 4;
+                c.p[k] = reinterpret_cast<void *>(h[k] + off * elem);
+            }
+            c.count = (uint32_t)(left < (size_t)chunk ? left : (size_t)chunk);
+            c.flags = flags;
+            c.tensor = (uint32_t)i;
+            chunks.push_back(c);
         }
         plan->total_elements += numel;
     }
@@ -136,10 +155,7 @@ static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanReque
         return nullptr;
     }
 
-    if (!hip_ok(hipMalloc(&plan->d_recs, recs.size() * sizeof(TensorRec)), "hipMalloc(recs)") ||
-        !hip_ok(hipMalloc(&plan->d_chunks, chunks.size() * sizeof(Chunk)), "hipMalloc(chunks)") ||
-        !hip_ok(hipMemcpyAsync(plan->d_recs, recs.data(), recs.size() * sizeof(TensorRec),
-                               hipMemcpyHostToDevice, ctx->stream), "upload recs") ||
+    if (!hip_ok(hipMalloc(&plan->d_chunks, chunks.size() * sizeof(Chunk)), "hipMalloc(chunks)") ||
         !hip_ok(hipMemcpyAsync(plan->d_chunks, chunks.data(), chunks.size() * sizeof(Chunk),
                                hipMemcpyHostToDevice, ctx->stream), "upload chunks") ||
         !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
@@ -192,119 +208,119 @@ __device__ inline void stream_store(T v, T *p)
     else *gp = v;
 }
 
-// Applies Rule to `count` elements starting at element `offset` of a tensor.
-// GradT is float or _Float16 (mixed precision: g = float(g16) * inv_scale and
-// an optional fp16 copy of the new weight is emitted).
-template <class Rule, bool NT, bool AMP>
-__device__ inline void process_chunk(const TensorRec &rec, uint64_t offset, uint32_t count,
-                                     const StepParams &prm, float inv_scale)
+template <class T, int N>
+struct VecOf {
+    typedef T type __attribute__((ext_vector_type(N)));
+};
+template <class T>
+struct VecOf<T, 1> {
+    typedef T type;
+};
+
+template <int N, class V>
+__device__ inline auto lane_of(const V &v, int c)
+{
+    if constexpr (N == 1) return v;
+    else return v[c];
+}
+
+template <int N, class V, class T>
+__device__ inline void set_lane(V &v, int c, T x)
+{
+    if constexpr (N == 1) v = x;
+    else v[c] = x;
+}
+
+// One lane's share of a slice: elements [first, first + N) of the chunk's
+// streams, N = VEC when the whole group is inside the chunk and the streams
+// are aligned for it, else 1.
+template <class Rule, int N, bool NT, bool AMP>
+__device__ inline void update_group(const Chunk &ch, uint32_t first, const StepParams &prm,
+                                    float inv_scale)
 {
     constexpr int NS = Rule::NSTATE;
     constexpr int NSA = NS > 0 ? NS : 1;
-    float *__restrict__ w = reinterpret_cast<float *>(rec.p[kSlotWeight]) + offset;
-    const float *__restrict__ g32 = nullptr;
-    const _Float16 *__restrict__ g16 = nullptr;
-    _Float16 *__restrict__ w16 = nullptr;
-    if (AMP) {
-        g16 = reinterpret_cast<const _Float16 *>(rec.p[kSlotGrad]) + offset;
-        if (rec.p[kSlotWeight16]) w16 = reinterpret_cast<_Float16 *>(rec.p[kSlotWeight16]) + offset;
-    } else {
-        g32 = reinterpret_cast<const float *>(rec.p[kSlotGrad]) + offset;
-    }
-    float *__restrict__ st[NSA];
-#pragma unroll
-    for (int k = 0; k < NS; k++) st[k] = reinterpret_cast<float *>(rec.p[kSlotState0 + k]) + offset;
+    typedef typename VecOf<float, N>::type FV;
+    typedef typename VecOf<_Float16, N>::type HV;
 
-    uint32_t done = 0;
-    if (rec.flags & kRecVectorOk) {
-        const uint32_t n4 = count >> 2;
-        floatx4 *w4 = reinterpret_cast<floatx4 *>(w);
-        for (uint32_t base = threadIdx.x; base < n4; base += kBlock * kUnroll) {
-            floatx4 W[kUnroll], G[kUnroll], S[NSA][kUnroll];
-            // all loads first: (2 + NS) * kUnroll independent 16-byte requests per lane
+    FV *wp = reinterpret_cast<FV *>(reinterpret_cast<float *>(ch.p[kSlotWeight]) + first);
+    FV W = stream_load<NT>(wp);
+    FV G;
+    if (AMP) {
+        HV h = stream_load<NT>(reinterpret_cast<const HV *>(
+            reinterpret_cast<const _Float16 *>(ch.p[kSlotGrad]) + first));
 #pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
-                const uint32_t i = base + u * kBlock;
-                if (i < n4) {
-                    W[u] = stream_load<NT>(w4 + i);
-                    if (AMP) {
-                        halfx4 h = stream_load<NT>(reinterpret_cast<const halfx4 *>(g16) + i);
-                        G[u] = floatx4{(float)h.x, (float)h.y, (float)h.z, (float)h.w};
-                    } else {
-                        G[u] = stream_load<NT>(reinterpret_cast<const floatx4 *>(g32) + i);
-                    }
-#pragma unroll
-                    for (int k = 0; k < NS; k++)
-                        S[k][u] = stream_load<NT>(reinterpret_cast<const floatx4 *>(st[k]) + i);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
-                const uint32_t i = base + u * kBlock;
-                if (i < n4) {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        float wv = W[u][c];
-                        float gv = G[u][c];
-                        if (AMP) gv = gv * inv_scale;
-                        float sv[NSA];
-#pragma unroll
-                        for (int k = 0; k < NS; k++) sv[k] = S[k][u][c];
-                        Rule::apply(wv, gv, sv, prm);
-                        W[u][c] = wv;
-#pragma unroll
-                        for (int k = 0; k < NS; k++) S[k][u][c] = sv[k];
-                    }
-                    stream_store<NT>(W[u], w4 + i);
-#pragma unroll
-                    for (int k = 0; k < NS; k++)
-                        stream_store<NT>(S[k][u], reinterpret_cast<floatx4 *>(st[k]) + i);
-                    if (AMP && w16) {
-                        halfx4 h = {(_Float16)W[u].x, (_Float16)W[u].y, (_Float16)W[u].z, (_Float16)W[u].w};
-                        stream_store<NT>(h, reinterpret_cast<halfx4 *>(w16) + i);
-                    }
-                }
-            }
-        }
-        done = n4 << 2;
+        for (int c = 0; c < N; c++) set_lane<N>(G, c, (float)lane_of<N>(h, c));
+    } else {
+        G = stream_load<NT>(reinterpret_cast<const FV *>(
+            reinterpret_cast<const float *>(ch.p[kSlotGrad]) + first));
     }
-    // scalar path: the < 4 element tail, or the whole chunk when a stream is misaligned
-    for (uint32_t i = done + threadIdx.x; i < count; i += kBlock) {
-        float wv = stream_load<false>(w + i);
-        float gv = AMP ? (float)stream_load<false>(g16 + i) * inv_scale : stream_load<false>(g32 + i);
+    FV S[NSA];
+    FV *sp[NSA];
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        sp[k] = reinterpret_cast<FV *>(reinterpret_cast<float *>(ch.p[kSlotState0 + k]) + first);
+        S[k] = stream_load<NT>(sp[k]);
+    }
+#pragma unroll
+    for (int c = 0; c < N; c++) {
+        float wv = lane_of<N>(W, c);
+        float gv = lane_of<N>(G, c);
+        if (AMP) gv = gv * inv_scale;
         float sv[NSA];
 #pragma unroll
-        for (int k = 0; k < NS; k++) sv[k] = stream_load<false>(st[k] + i);
+        for (int k = 0; k < NS; k++) sv[k] = lane_of<N>(S[k], c);
         Rule::apply(wv, gv, sv, prm);
-        stream_store<false>(wv, w + i);
+        set_lane<N>(W, c, wv);
 #pragma unroll
-        for (int k = 0; k < NS; k++) stream_store<false>(sv[k], st[k] + i);
-        if (AMP && w16) stream_store<false>((_Float16)wv, w16 + i);
+        for (int k = 0; k < NS; k++) set_lane<N>(S[k], c, sv[k]);
+    }
+    stream_store<NT>(W, wp);
+#pragma unroll
+    for (int k = 0; k < NS; k++) stream_store<NT>(S[k], sp[k]);
+    if (AMP && ch.p[kSlotWeight16]) {
+        HV h;
+#pragma unroll
+        for (int c = 0; c < N; c++) set_lane<N>(h, c, (_Float16)lane_of<N>(W, c));
+        stream_store<NT>(h, reinterpret_cast<HV *>(reinterpret_cast<_Float16 *>(ch.p[kSlotWeight16]) + first));
     }
 }
 
-template <class Rule, bool NT>
-__global__ void __launch_bounds__(kBlock)
-multi_tensor_update_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
-                           StepParams prm)
+// Workgroup b -> (chunk, slice).  slice_shift = log2(slices per chunk).
+template <class Rule, int VEC, bool NT, bool AMP>
+__device__ inline void update_slice(const Chunk &ch, uint32_t slice_shift, const StepParams &prm,
+                                    float inv_scale)
 {
-    const Chunk ch = chunks[blockIdx.x];
-    const TensorRec rec = recs[ch.tensor];
-    process_chunk<Rule, NT, false>(rec, ch.offset, ch.count, prm, 1.0f);
+    const uint32_t slice = blockIdx.x & ((1u << slice_shift) - 1u);
+    const uint32_t local = (slice * kBlock + threadIdx.x) * VEC;   // first element of this lane within the chunk
+    if (local >= ch.count) return;
+    constexpr uint32_t vec_flag = VEC == 4 ? kRecVec4Ok : kRecVec2Ok;
+    if (VEC > 1 && (ch.flags & vec_flag) && local + VEC <= ch.count) {
+        update_group<Rule, VEC, NT, AMP>(ch, local, prm, inv_scale);
+    } else {
+        const uint32_t n = ch.count - local < (uint32_t)VEC ? ch.count - local : (uint32_t)VEC;
+        for (uint32_t e = 0; e < n; e++) update_group<Rule, 1, NT, AMP>(ch, local + e, prm, inv_scale);
+    }
+}
+
+template <class Rule, int VEC, bool NT>
+__global__ void __launch_bounds__(kBlock)
+multi_tensor_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm)
+{
+    const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    update_slice<Rule, VEC, NT, false>(ch, slice_shift, prm, 1.0f);
 }
 
 // SGD: a tensor without a momentum buffer takes the vanilla rule.
-template <bool NT>
+template <int VEC, bool NT>
 __global__ void __launch_bounds__(kBlock)
-multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
-                        StepParams prm)
+multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm)
 {
-    const Chunk ch = chunks[blockIdx.x];
-    const TensorRec rec = recs[ch.tensor];
-    if (prm.momentum > 0.0f && rec.p[kSlotState0] != nullptr)
-        process_chunk<SgdMomentumRule, NT, false>(rec, ch.offset, ch.count, prm, 1.0f);
+    const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    if (prm.momentum > 0.0f && ch.p[kSlotState0] != nullptr)
+        update_slice<SgdMomentumRule, VEC, NT, false>(ch, slice_shift, prm, 1.0f);
     else
-        process_chunk<SgdVanillaRule, NT, false>(rec, ch.offset, ch.count, prm, 1.0f);
+        update_slice<SgdVanillaRule, VEC, NT, false>(ch, slice_shift, prm, 1.0f);
 }
 
 // ---- mixed precision ----
@@ -326,27 +342,25 @@ struct AmpDeviceState {
 // one atomic per workgroup that saw a hit.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
-amp_overflow_check_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
-                          AmpDeviceState *__restrict__ state)
+amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state)
 {
     __shared__ unsigned int wave_hit[kBlock / 64];
     const Chunk ch = chunks[blockIdx.x];
-    const TensorRec rec = recs[ch.tensor];
-    const unsigned short *g = reinterpret_cast<const unsigned short *>(rec.p[kSlotGrad]) + ch.offset;
+    const unsigned short *g = reinterpret_cast<const unsigned short *>(ch.p[kSlotGrad]);
     unsigned int bad = 0;
     uint32_t done = 0;
-    if (rec.flags & kRecGrad16VectorOk) {
+    if (ch.flags & kRecGrad16VectorOk) {
         const uint32_t n8 = ch.count >> 3;
         const uintx4 *g8 = reinterpret_cast<const uintx4 *>(g);
-        for (uint32_t base = threadIdx.x; base < n8; base += kBlock * kUnroll) {
-            uintx4 v[kUnroll];
+        for (uint32_t base = threadIdx.x; base < n8; base += kBlock * kCheckUnroll) {
+            uintx4 v[kCheckUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
+            for (int u = 0; u < kCheckUnroll; u++) {
                 const uint32_t i = base + u * kBlock;
                 v[u] = (i < n8) ? stream_load<NT>(g8 + i) : uintx4{0u, 0u, 0u, 0u};
             }
 #pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
+            for (int u = 0; u < kCheckUnroll; u++) {
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     const unsigned int e = v[u][c] & 0x7C007C00u;
@@ -357,7 +371,7 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, const TensorRec *__r
         done = n8 << 3;
     }
     for (uint32_t i = done + threadIdx.x; i < ch.count; i += kBlock)
-        bad |= ((g[i] & 0x7C00u) == 0x7C00u);
+        bad |= ((stream_load<false>(g + i) & 0x7C00u) == 0x7C00u);
 
     const unsigned long long ballot = __ballot(bad != 0);
     if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = (ballot != 0ull);
@@ -372,16 +386,15 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, const TensorRec *__r
 
 // Phase B: the Adam update on unscaled gradients, skipped as a whole when the
 // flag is set.
-template <bool NT>
+template <int VEC, bool NT>
 __global__ void __launch_bounds__(kBlock)
-amp_adam_update_kernel(const Chunk *__restrict__ chunks, const TensorRec *__restrict__ recs,
-                       StepParams prm, const AmpDeviceState *__restrict__ state)
+amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
+                       const AmpDeviceState *__restrict__ state)
 {
     if (state->found_inf) return;
     const float inv_scale = 1.0f / state->scale;
-    const Chunk ch = chunks[blockIdx.x];
-    const TensorRec rec = recs[ch.tensor];
-    process_chunk<AdamRule, NT, true>(rec, ch.offset, ch.count, prm, inv_scale);
+    const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    update_slice<AdamRule, VEC, NT, true>(ch, slice_shift, prm, inv_scale);
 }
 
 // Epilogue (one lane, same stream, after phase B has drained): advances the
@@ -454,16 +467,42 @@ static int prepare(uintptr_t device, const PlanRequest &req, int hip_error_code,
     return 0;
 }
 
+// Grid size: every chunk gets the same number of slices; the slices past the
+// end of a short chunk exit at once.
+static bool launch_geometry(const MultiTensorPlan &plan, int vec, uint32_t &grid, uint32_t &shift)
+{
+    shift = slice_shift_for(plan.chunk_elements, vec);
+    const uint64_t blocks = (uint64_t)plan.num_chunks << shift;
+    if (blocks > 0x7FFFFFFFull) {
+        set_error("parameter list needs %llu workgroups, more than one launch can address",
+                  (unsigned long long)blocks);
+        return false;
+    }
+    grid = (uint32_t)blocks;
+    return true;
+}
+
+template <class Rule, int VEC>
+static void launch_rule_vec(const Launch &l, const StepParams &prm, uint32_t grid, uint32_t shift)
+{
+    if (current_nontemporal())
+        multi_tensor_update_kernel<Rule, VEC, true><<<grid, kBlock, 0, l.ctx->stream>>>(
+            l.plan->d_chunks, shift, prm);
+    else
+        multi_tensor_update_kernel<Rule, VEC, false><<<grid, kBlock, 0, l.ctx->stream>>>(
+            l.plan->d_chunks, shift, prm);
+}
+
 template <class Rule>
 static int launch_rule(const Launch &l, const StepParams &prm, int hip_error_code)
 {
     if (l.plan->num_chunks == 0) return 0;
-    if (current_nontemporal())
-        multi_tensor_update_kernel<Rule, true><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
-            l.plan->d_chunks, l.plan->d_recs, prm);
-    else
-        multi_tensor_update_kernel<Rule, false><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
-            l.plan->d_chunks, l.plan->d_recs, prm);
+    const int vec = current_vec();
+    uint32_t grid, shift;
+    if (!launch_geometry(*l.plan, vec, grid, shift)) return hip_error_code;
+    if (vec == 4) launch_rule_vec<Rule, 4>(l, prm, grid, shift);
+    else if (vec == 2) launch_rule_vec<Rule, 2>(l, prm, grid, shift);
+    else launch_rule_vec<Rule, 1>(l, prm, grid, shift);
     return hip_ok(hipGetLastError(), "update kernel launch") ? 0 : hip_error_code;
 }
 
@@ -535,16 +574,18 @@ float gm_nadam_mu_next(float beta1, int step_count)
     return beta1 * one_minus;
 }
 
-int gm_set_tuning(int chunk_elements, int nontemporal)
+int gm_set_tuning(int chunk_elements, int nontemporal, int vec)
 {
-    if (chunk_elements != 0) {
-        if (chunk_elements < 1024 || chunk_elements % 1024 != 0) return -1;
-        g_chunk_elements.store(chunk_elements);
-    } else {
-        g_chunk_elements.store(kDefaultChunkElements);
-    }
-    if (nontemporal >= 0) g_nontemporal.store(nontemporal ? 1 : 0);
-    else g_nontemporal.store(1);
+    const int v = vec == 0 ? kDefaultVec : vec;
+    const int c = chunk_elements == 0 ? kDefaultChunkElements : chunk_elements;
+    if (v != 1 && v != 2 && v != 4) return -1;
+    // a chunk is a power-of-two number of 256 * vec element slices
+    if (c < kBlock * v || c % (kBlock * v) != 0) return -1;
+    const int slices = c / (kBlock * v);
+    if ((slices & (slices - 1)) != 0) return -1;
+    g_vec.store(v);
+    g_chunk_elements.store(c);
+    g_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
     return 0;
 }
 
@@ -572,12 +613,16 @@ int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     p.momentum = momentum;
     p.weight_decay = weight_decay;
     p.nesterov = nesterov;
-    if (current_nontemporal())
-        multi_tensor_sgd_kernel<true><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
-            l.plan->d_chunks, l.plan->d_recs, p);
-    else
-        multi_tensor_sgd_kernel<false><<<l.plan->num_chunks, kBlock, 0, l.ctx->stream>>>(
-            l.plan->d_chunks, l.plan->d_recs, p);
+    const int vec = current_vec();
+    const bool nt = current_nontemporal();
+    uint32_t grid, shift;
+    if (!launch_geometry(*l.plan, vec, grid, shift)) return -10;
+    hipStream_t st = l.ctx->stream;
+#define GM_LAUNCH_SGD(V, N) multi_tensor_sgd_kernel<V, N><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, shift, p)
+    if (vec == 4) { if (nt) GM_LAUNCH_SGD(4, true); else GM_LAUNCH_SGD(4, false); }
+    else if (vec == 2) { if (nt) GM_LAUNCH_SGD(2, true); else GM_LAUNCH_SGD(2, false); }
+    else { if (nt) GM_LAUNCH_SGD(1, true); else GM_LAUNCH_SGD(1, false); }
+#undef GM_LAUNCH_SGD
     return hip_ok(hipGetLastError(), "sgd kernel launch") ? 0 : -10;
 }
 
@@ -866,17 +911,17 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
     const uint32_t chunks = l.plan->num_chunks;
     hipStream_t st = l.ctx->stream;
     if (chunks > 0) {
-        if (current_nontemporal()) {
-            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs,
-                                                                      amp->d_state);
-            amp_adam_update_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, p,
-                                                                   amp->d_state);
-        } else {
-            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs,
-                                                                       amp->d_state);
-            amp_adam_update_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, l.plan->d_recs, p,
-                                                                    amp->d_state);
-        }
+        const int vec = current_vec();
+        const bool nt = current_nontemporal();
+        uint32_t grid, shift;
+        if (!launch_geometry(*l.plan, vec, grid, shift)) return -6;
+        if (nt) amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
+        else amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
+#define GM_LAUNCH_AMP(V, N) amp_adam_update_kernel<V, N><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, shift, p, amp->d_state)
+        if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true); else GM_LAUNCH_AMP(4, false); }
+        else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true); else GM_LAUNCH_AMP(2, false); }
+        else { if (nt) GM_LAUNCH_AMP(1, true); else GM_LAUNCH_AMP(1, false); }
+#undef GM_LAUNCH_AMP
     }
     amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state);
     if (!hip_ok(hipGetLastError(), "mixed-precision kernel launch")) return -6;

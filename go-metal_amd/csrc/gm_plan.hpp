@@ -1,14 +1,16 @@
 // Multi-tensor launch plan: the device-side tables one update launch walks.
 //
 // A step over a parameter list is ONE kernel launch.  The host flattens the
-// list into fixed-size chunks; workgroup b processes chunk b.  Two small tables
-// live in HBM and are rebuilt only when the caller's handles change:
+// list into fixed-size chunks; a chunk is shared by a fixed number of
+// consecutive workgroups (one slice each).  One table lives in HBM and is
+// rebuilt only when the caller's handles change:
 //
-//   TensorRec recs[num_tensors]   base addresses of every stream of a tensor
-//   Chunk     chunks[num_chunks]  {tensor index, element offset, element count}
+//   Chunk chunks[num_chunks]   the address of the chunk's first element in
+//                              every stream, the element count and flags
 //
-// Both are read with wave-uniform (scalar) loads, so they cost one cache line
-// per workgroup against >= 100 KB of streamed data.
+// A descriptor is one 64-byte line, fetched by a single wave-uniform (scalar)
+// load that hits in cache for all but the first workgroup of the chunk
+// (64 bytes of table per 16384 elements, i.e. per >= 320 KB of streamed data).
 #pragma once
 
 #include "gm_context.hpp"
@@ -27,23 +29,19 @@ enum : int {
 };
 
 enum : uint32_t {
-    kRecVectorOk = 1u,       // every used stream is aligned for 16-byte (fp32) / 8-byte (fp16) lanes
-    kRecGrad16VectorOk = 2u, // the fp16 gradient is 16-byte aligned (overflow-check kernel)
+    kRecVec2Ok = 1u,         // every used stream is aligned for 2-element lanes (8 B fp32 / 4 B fp16)
+    kRecVec4Ok = 2u,         // ... for 4-element lanes (16 B fp32 / 8 B fp16)
+    kRecGrad16VectorOk = 4u, // the fp16 gradient is 16-byte aligned (overflow-check kernel)
 };
 
-struct TensorRec {
-    void *p[kNumSlots];
+struct alignas(64) Chunk {
+    void *p[kNumSlots];   // first element of this chunk in each stream (nullptr: stream unused)
+    uint32_t count;       // elements in this chunk (<= chunk_elements)
     uint32_t flags;
+    uint32_t tensor;      // index into the caller's list (diagnostics only)
     uint32_t pad;
 };
-static_assert(sizeof(TensorRec) == 56, "TensorRec layout");
-
-struct Chunk {
-    uint32_t tensor;
-    uint32_t count;     // elements in this chunk (<= chunk_elements)
-    uint64_t offset;    // first element, multiple of chunk_elements
-};
-static_assert(sizeof(Chunk) == 16, "Chunk layout");
+static_assert(sizeof(Chunk) == 64, "Chunk layout");
 
 // Which update rule a plan (and its validation) was built for.
 enum RuleKind : int {
@@ -67,7 +65,6 @@ struct MultiTensorPlan {
     std::vector<int> sizes;
     // ---- result ----
     int status = 0;              // validation result: 0 or the entry point's error code
-    TensorRec *d_recs = nullptr;
     Chunk *d_chunks = nullptr;
     uint32_t num_chunks = 0;
     uint64_t total_elements = 0;
@@ -95,9 +92,11 @@ struct PlanRequest {
 // the caller holds).  nullptr on a HIP failure (error already recorded).
 MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req);
 
-// Elements per workgroup chunk currently in force (tunable for sweeps).
+// Elements per chunk currently in force (tunable for sweeps).
 int current_chunk_elements();
 // Whether streaming accesses carry the non-temporal hint.
 bool current_nontemporal();
+// fp32 elements per lane (1, 2 or 4).
+int current_vec();
 
 }  // namespace gm

@@ -128,10 +128,11 @@ def test_config3_ragged_25m(dev, config3_data, rule, hyper):
 ])
 def test_variants_and_ragged_edges(dev, rule, hyper):
     """Every rule variant over sizes that exercise the vector body, the scalar tail, one-element
-    tensors, an empty tensor and chunk boundaries (a workgroup chunk is 4096 elements)."""
+    tensors, an empty tensor, workgroup-slice boundaries (256 elements) and chunk boundaries
+    (16384 elements)."""
     rng = np.random.default_rng(99)
-    sizes = [1, 2, 3, 4, 5, 0, 63, 64, 65, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8193, 65535, 65537, 131072 + 7,
-             300001]
+    sizes = [1, 2, 3, 4, 5, 0, 63, 64, 65, 255, 256, 257, 1023, 1025, 4095, 4097, 16383, 16384, 16385, 65535, 65537,
+             131072 + 7, 300001]
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
     run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
              steps=6, check_every=3, nthreads=1)
