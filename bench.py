@@ -32,6 +32,10 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
                    "adam_amp": 28}
 
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
+# file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
+MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8400e10}
+
 from workloads import amp_125m_sizes, cnn_sizes, ragged_sizes, transformer_block_sizes  # noqa: E402
 
 WORKLOADS = {
@@ -179,11 +183,7 @@ def main():
     dev.free(src)
     dev.free(dst)
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get(f"{args.workload}:{rule}")
+    traffic = MEASURED_HBM_TRAFFIC.get((args.workload, rule))
 
     result = {
         "metric": "params updated/sec (Adam fp32 multi-tensor step) + achieved HBM GB/s (% of peak)"

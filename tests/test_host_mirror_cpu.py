@@ -1,0 +1,211 @@
+"""Host-side mirror of the Go `optimizer` and `memory` packages: the behaviour the reference's
+own GPU-less tests pin (mock optimizers, helper tables, pool maths), driven through
+include/gometal_optimizer.h.  No GPU is needed: nothing here reaches a kernel."""
+import json
+import math
+
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+
+pkg = load_package()
+lib = pkg.load_library()
+MOCK_DEVICE = 0x1000      # memory.CreateMockDevice, memory/manager.go:322-326
+MOCK_QUEUE = 0x2000
+
+
+def f32(x):
+    return float(np.float32(x))
+
+
+@pytest.fixture
+def mm():
+    h = lib.gmo_memory_manager_new(MOCK_DEVICE)
+    yield h
+    lib.gmo_memory_manager_free(h)
+
+
+def new(kind, config, shapes, mm, device=MOCK_DEVICE):
+    return pkg.HostOptimizer(kind, config, shapes, mm, device)
+
+
+# ---- config defaults: adam_test.go:129-153, sgd_test.go:13-38, rmsprop.go:54-63, adagrad.go:42-48,
+# ---- adadelta.go:43-49, nadam.go:47-55
+@pytest.mark.parametrize("kind,expected", [
+    ("sgd", [0.01, 0.0, 0.0, 0.0]),
+    ("adam", [0.001, 0.9, 0.999, 1e-8, 0.0]),
+    ("rmsprop", [0.01, 0.99, 1e-8, 0.0, 0.0, 0.0]),
+    ("adagrad", [0.01, 1e-10, 0.0]),
+    ("adadelta", [0.95, 1e-6, 0.0]),
+    ("nadam", [0.002, 0.9, 0.999, 1e-8, 0.0]),
+])
+def test_default_configs(kind, expected):
+    import ctypes
+    cfg = (ctypes.c_float * 6)()
+    n = lib.gmo_default_config(pkg.KINDS[kind], cfg)
+    assert n == len(expected)
+    assert [cfg[k] for k in range(n)] == [f32(v) for v in expected]
+
+
+# ---- constructor validation, in the order and with the strings of the Go constructors
+def test_constructor_argument_errors(mm):
+    for kind, cfg in [("sgd", [0.01, 0, 0, 0]), ("adam", [1e-3, .9, .999, 1e-8, 0]),
+                      ("rmsprop", [.01, .99, 1e-8, 0, 0, 0]), ("adagrad", [.01, 1e-10, 0]),
+                      ("adadelta", [.95, 1e-6, 0]), ("nadam", [.002, .9, .999, 1e-8, 0])]:
+        assert new(kind, cfg, [[4]], 0).error == "memory manager cannot be nil"
+        assert new(kind, cfg, [[4]], mm, device=0).error == "device cannot be nil"
+        assert new(kind, cfg, [], mm).error == "no weight shapes provided"
+
+
+def test_sgd_validation_messages(mm):                       # sgd.go:77-88
+    assert new("sgd", [-0.01, 0, 0, 0], [[4]], mm).error == "learning rate cannot be negative: -0.010000"
+    assert new("sgd", [0.01, -0.5, 0, 0], [[4]], mm).error == "momentum cannot be negative: -0.500000"
+    assert new("sgd", [0.01, 1.5, 0, 0], [[4]], mm).error == "momentum cannot be greater than 1.0: 1.500000"
+    assert new("sgd", [0.01, 0, -1, 0], [[4]], mm).error == "weight decay cannot be negative: -1.000000"
+
+
+def test_adadelta_and_nadam_validation_messages(mm):        # adadelta.go:70-72, nadam.go:77-91
+    assert new("adadelta", [0.0, 1e-6, 0], [[4]], mm).error == "rho must be in range (0, 1), got 0.000000"
+    assert new("adadelta", [1.0, 1e-6, 0], [[4]], mm).error == "rho must be in range (0, 1), got 1.000000"
+    assert new("nadam", [0.0, .9, .999, 1e-8, 0], [[4]], mm).error == "learning rate must be positive, got 0.000000"
+    assert new("nadam", [.002, 1.0, .999, 1e-8, 0], [[4]], mm).error == "beta1 must be in [0, 1), got 1.000000"
+    assert new("nadam", [.002, .9, -0.1, 1e-8, 0], [[4]], mm).error == "beta2 must be in [0, 1), got -0.100000"
+    assert new("nadam", [.002, .9, .999, 0.0, 0], [[4]], mm).error == "epsilon must be positive, got 0.000000e+00"
+    assert new("nadam", [.002, .9, .999, 1e-8, -1], [[4]], mm).error == "weight decay must be non-negative, got -1.000000"
+
+
+@pytest.fixture
+def vanilla_sgd(mm):
+    """SGD without momentum allocates nothing, so it can be built without a GPU
+    (the reference's MockSGDOptimizer, sgd_test.go)."""
+    opt = new("sgd", [0.01, 0.0, 0.0, 0], [[10, 5], [5]], mm)
+    assert opt.error is None
+    yield opt
+    opt.free()
+
+
+def test_set_weight_buffers_length_check(vanilla_sgd):      # sgd.go:151-158
+    assert vanilla_sgd.SetWeightBuffers([0x1000]) == "expected 2 weight buffers, got 1"
+    assert vanilla_sgd.SetWeightBuffers([0x1000, 0x2000]) is None
+
+
+def test_step_errors_and_step_count(vanilla_sgd):           # sgd_test.go:694-720
+    vanilla_sgd.SetWeightBuffers([0x1000, 0x2000])
+    err = vanilla_sgd.Step([0x1000])
+    assert err == "gradient buffers length (1) doesn't match weight buffers length (2)"
+    assert vanilla_sgd.GetStepCount() == 0
+    # right count, but no GPU behind the mock device: the native step fails, the count stays incremented
+    err = vanilla_sgd.Step([0x1000, 0x2000])
+    if err is not None:
+        assert err.startswith("SGD step execution failed: SGD step execution failed with error code: ")
+    assert vanilla_sgd.GetStepCount() == 1
+
+
+def test_set_command_pool_and_learning_rate(vanilla_sgd):   # adam_test.go:257-279, sgd.go:191-199
+    assert lib.gmo_uses_pooling(vanilla_sgd.handle) == 0
+    vanilla_sgd.SetCommandPool(MOCK_QUEUE)
+    assert lib.gmo_uses_pooling(vanilla_sgd.handle) == 1
+    vanilla_sgd.SetCommandPool(0)
+    assert lib.gmo_uses_pooling(vanilla_sgd.handle) == 0
+    vanilla_sgd.UpdateLearningRate(0.5)
+    assert vanilla_sgd.field("LearningRate") == 0.5
+
+
+def test_get_state_structure_without_buffers(vanilla_sgd):  # sgd.go:229-256
+    text, err = vanilla_sgd.GetStateJSON()
+    assert err is None
+    st = json.loads(text)
+    assert st["type"] == "SGD" and st["state_data"] == []
+    assert set(st["parameters"]) == {"learning_rate", "momentum", "weight_decay", "nesterov", "step_count"}
+    assert st["parameters"]["nesterov"] is False and st["parameters"]["step_count"] == 0
+    assert np.float32(st["parameters"]["learning_rate"]) == np.float32(0.01)
+
+
+def test_load_state_validation_and_tolerance(vanilla_sgd):  # adam_test.go:339-454 restated for SGD
+    sgd = vanilla_sgd
+    assert sgd.LoadStateJSON(json.dumps({"type": "InvalidType", "parameters": {}, "state_data": []})) == \
+        "state type mismatch: expected SGD, got InvalidType"
+    ok = {"type": "SGD", "parameters": {"learning_rate": 0.002, "momentum": 0.85, "weight_decay": 0.005,
+                                        "nesterov": True, "step_count": 10}, "state_data": []}
+    assert sgd.LoadStateJSON(json.dumps(ok)) is None
+    assert sgd.field("LearningRate") == f32(0.002) and sgd.field("Momentum") == f32(0.85)
+    assert sgd.field("WeightDecay") == f32(0.005) and sgd.field("Nesterov") == 1.0
+    assert sgd.GetStepCount() == 10
+    # missing parameters leave the fields alone
+    assert sgd.LoadStateJSON(json.dumps({"type": "SGD", "parameters": {"learning_rate": 0.003}})) is None
+    assert sgd.field("LearningRate") == f32(0.003) and sgd.field("Momentum") == f32(0.85)
+    # wrong types are ignored, not errors
+    assert sgd.LoadStateJSON(json.dumps({"type": "SGD", "parameters": {"learning_rate": "not_a_number",
+                                                                      "momentum": 0.9}})) is None
+    assert sgd.field("LearningRate") == f32(0.003) and sgd.field("Momentum") == f32(0.9)
+    # a momentum tensor for an optimizer that has no momentum buffers (sgd.go:281-283)
+    bad = {"type": "SGD", "parameters": {}, "state_data": [
+        {"name": "momentum_0", "shape": [50], "data": [0.0] * 50, "state_type": "momentum"}]}
+    assert sgd.LoadStateJSON(json.dumps(bad)) == "momentum buffer 0 not allocated"
+    bad["state_data"][0]["name"] = "momentum_7"
+    assert sgd.LoadStateJSON(json.dumps(bad)) == "invalid buffer index in tensor name: momentum_7"
+    assert sgd.LoadStateJSON("{not json") .startswith("invalid optimizer state JSON")
+
+
+def test_cleanup_clears_lists(vanilla_sgd):                 # sgd.go:212-226
+    vanilla_sgd.Cleanup()
+    assert vanilla_sgd.SetWeightBuffers([0x1000, 0x2000]) == "expected 0 weight buffers, got 2"
+
+
+# ---- helper tables
+@pytest.mark.parametrize("name,expected", [                  # state_helpers_test.go:316-365
+    ("momentum_0", 0), ("variance_5", 5), ("squared_grad_avg_10", 10), ("momentum", -1),
+    ("momentum_abc", -1), ("", -1), ("_", -1), ("momentum_buffer_5", 5), ("momentum_-1", -1),
+    ("momentum_999", 999)])
+def test_extract_buffer_index(name, expected):
+    assert lib.gmo_extract_buffer_index(name.encode()) == expected
+
+
+@pytest.mark.parametrize("shape,expected", [                 # state_helpers_test.go:212-246
+    ([], 1), ([10], 10), ([10, 20], 200), ([5, 10, 20], 1000), ([2, 3, 4, 5], 120), ([1], 1), ([0], 0)])
+def test_calculate_tensor_size(shape, expected):
+    assert lib.gmo_calculate_tensor_size(pkg.int_array(shape) if shape else None, len(shape)) == expected
+
+
+# ---- package memory
+@pytest.mark.parametrize("requested,expected", [(100, 1024), (1024, 1024), (5000, 16384),
+                                                (100000000, 100000000)])   # memory_test.go:219-227
+def test_find_pool_size(mm, requested, expected):
+    assert lib.gmo_find_pool_size(mm, requested) == expected
+
+
+@pytest.mark.parametrize("size,expected", [(1024, 100), (4096, 100), (16384, 50), (65536, 50), (262144, 20),
+                                           (1048576, 20), (4194304, 20), (16777216, 20), (67108864, 15)])
+def test_reference_pool_caps_table(size, expected):           # memory_test.go:242-255
+    assert lib.gmo_reference_max_pool_size(size) == expected
+    # the cap in force is never below the reference's, and a 1B-parameter Adam state fits
+    assert lib.gmo_calculate_max_pool_size(size) >= expected
+
+
+def test_pool_caps_hold_transformer_sized_state():
+    """28 tensors of 64 MB need 56 state buffers for Adam; the reference's cap of 15 refuses them."""
+    assert lib.gmo_reference_max_pool_size(67108864) < 56 <= lib.gmo_calculate_max_pool_size(67108864)
+    lib.gmo_set_pool_byte_budget(10 * 67108864)
+    try:
+        assert lib.gmo_calculate_max_pool_size(67108864) == 15      # budget below the reference cap: the cap wins
+        lib.gmo_set_pool_byte_budget(100 * 67108864)
+        assert lib.gmo_calculate_max_pool_size(67108864) == 100
+    finally:
+        lib.gmo_set_pool_byte_budget(128 << 30)
+
+
+def test_allocate_without_global_manager_or_gpu_returns_nil(mm):   # manager.go:289-296
+    # no global manager yet in this process (or no GPU behind it): AllocateBuffer signals failure by nil
+    assert lib.gmo_allocate_buffer(mm, 1024) == 0 or lib.create_metal_device() != 0
+    lib.gmo_release_buffer(mm, 0)      # nil is ignored
+
+
+def test_optimizer_state_json_round_trip_is_exact():
+    """float32 values survive ToJSON -> FromJSON bit for bit (9 significant digits)."""
+    rng = np.random.default_rng(5)
+    vals = np.concatenate([rng.standard_normal(200).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 200),
+                           np.array([0.0, -0.0, 1e-45, 3.4028235e38, 1.17549435e-38], np.float32)]).astype(np.float32)
+    for v in vals:
+        assert np.float32(float("%.9g" % float(v))) == v or (v == 0)
+    assert not math.isnan(vals.sum())
