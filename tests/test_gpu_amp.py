@@ -1,0 +1,180 @@
+"""Mixed-precision Adam on the GPU against the CPU oracle: the skip / loss-scale sequence must be
+bit-exact over the whole run; weights, moments and the fp16 weight copy are held to 0 ulp."""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+
+from harness import amp_step_gpu, gpu_device
+from oracle_lib import oracle
+from workloads import amp_125m_sizes, transformer_block_sizes
+from __graft_entry__ import load_package
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "optimizer_kat.json")) as f:
+    KAT = json.load(f)
+NTHREADS = min(16, os.cpu_count() or 1)
+HYPER = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = gpu_device()
+    if d is None:
+        pytest.fail("libgometal_hip.so is missing or no GPU is usable: GPU tests cannot run")
+    return d
+
+
+class AmpPair:
+    """The same tensor list on the GPU (C ABI) and in the oracle."""
+
+    def __init__(self, dev, weights, hyper, amp_cfg=(65536.0, 2.0, 0.5, 2000), nthreads=1):
+        self.dev, self.pkg, self.h, self.nthreads = dev, load_package(), hyper, nthreads
+        self.sizes = [w.size for w in weights]
+        self.n = len(weights)
+        self.w = [np.array(w, np.float32, copy=True) for w in weights]
+        self.m = [np.zeros(s, np.float32) for s in self.sizes]
+        self.v = [np.zeros(s, np.float32) for s in self.sizes]
+        self.w16 = [np.zeros(s, np.uint16) for s in self.sizes]
+        self.st = oracle().amp_state(*amp_cfg)
+        self.d = {"w": [dev.from_numpy(w) for w in self.w],
+                  "m": [dev.alloc(4 * s, zero=True) for s in self.sizes],
+                  "v": [dev.alloc(4 * s, zero=True) for s in self.sizes],
+                  "w16": [dev.alloc(2 * s, zero=True) for s in self.sizes],
+                  "g16": [dev.alloc(2 * s) for s in self.sizes]}
+        self.c = {k: self.pkg.handle_array(v) for k, v in self.d.items()}
+        self.bs = self.pkg.int_array([4 * s for s in self.sizes])
+        self.amp = dev.lib.gm_amp_state_create(dev.handle, *amp_cfg)
+        assert self.amp
+        self.gpu_steps = 0
+
+    def step(self, g16, upload=True):
+        if upload:
+            for h, g in zip(self.d["g16"], g16):
+                self.dev.upload(h, g)
+        got = amp_step_gpu(self.dev, self.pkg, self.c, self.bs, self.n, self.h, self.gpu_steps + 1, self.amp)
+        if not got[0]:
+            self.gpu_steps += 1
+        want_skipped = oracle().adam_amp(self.w, g16, self.m, self.v, self.w16, state=self.st,
+                                         nthreads=self.nthreads, **self.h)
+        want = (want_skipped, float(np.float32(self.st.scale)), self.st.growth_tracker)
+        assert got == want, (got, want)
+        assert self.gpu_steps == self.st.step_count
+        return got[0]
+
+    def compare(self, context=""):
+        for name, host, dtype in (("w", self.w, np.float32), ("m", self.m, np.float32), ("v", self.v, np.float32),
+                                  ("w16", self.w16, np.uint16)):
+            for k, ref in enumerate(host):
+                got = self.dev.to_numpy(self.d[name][k], ref.size, dtype)
+                assert np.array_equal(got.view(np.uint8), ref.view(np.uint8)), (context, name, k)
+
+    def close(self):
+        self.dev.lib.gm_amp_state_destroy(self.amp)
+        for v in self.d.values():
+            for h in v:
+                self.dev.free(h)
+
+
+@pytest.mark.parametrize("case", KAT["amp_cases"], ids=[c["name"] for c in KAT["amp_cases"]])
+def test_amp_golden_vectors(dev, case):
+    h, a = case["hyper"], case["amp"]
+    w0 = [np.array(t, np.uint32).view(np.float32) for t in case["w0"]]
+    pair = AmpPair(dev, w0, h, (a["init_scale"], a["growth_factor"], a["backoff_factor"], a["growth_interval"]))
+    try:
+        for k, step in enumerate(case["g16"]):
+            skipped = pair.step([np.array(t, np.uint16) for t in step])
+            exp = case["expect"][k]
+            assert skipped == exp["skipped"]
+            for ti in range(pair.n):
+                assert dev.to_numpy(pair.d["w"][ti], pair.sizes[ti]).view(np.uint32).tolist() == exp["w"][ti]
+                assert dev.to_numpy(pair.d["w16"][ti], pair.sizes[ti], np.uint16).tolist() == exp["w16"][ti]
+    finally:
+        pair.close()
+
+
+def test_config4_skip_and_scale_sequence_5000_steps(dev):
+    """The 5000-step schedule of config 4 (60 tensors, loss scale 65536, backoff x0.5, growth x2
+    every 2000 clean steps, +-inf / NaN injected into one random element on a seeded 0.5 % of steps)
+    with every tensor at 1/1000 of its size, so the oracle keeps pace: every step's
+    (skipped, scale, clean-step counter, step count) must equal the oracle's, and p / m / v / fp16
+    copy are compared bit for bit every 500 steps."""
+    rng = np.random.default_rng(0x6D657461 + 4)
+    sizes = [max(1, s // 1000) for s in amp_125m_sizes()]
+    w = [rng.normal(0, 0.02, s).astype(np.float32) for s in sizes]
+    pool = [[rng.normal(0, 1e-4, s).astype(np.float32) for s in sizes] for _ in range(8)]
+    inject = rng.random(5000) < 0.005
+    pair = AmpPair(dev, w, HYPER)
+    skipped_total = 0
+    try:
+        for k in range(5000):
+            scale = np.float32(pair.st.scale)
+            g16 = [(g * scale).astype(np.float16).view(np.uint16) for g in pool[k % len(pool)]]
+            if inject[k]:
+                t = int(rng.integers(0, len(sizes)))
+                g16[t][int(rng.integers(0, sizes[t]))] = [0x7C00, 0xFC00, 0x7E00][skipped_total % 3]
+            skipped_total += pair.step(g16)
+            if (k + 1) % 500 == 0:
+                pair.compare(f"step {k + 1}")
+        assert skipped_total == int(inject.sum()) and skipped_total > 10
+        assert pair.st.step_count == 5000 - skipped_total
+    finally:
+        pair.close()
+
+
+def device_normal_f16(dev, sizes, seed, std, scale):
+    """fp16 gradient tensors generated on the device; returns (handles, host copies)."""
+    handles, host = [], []
+    for k, s in enumerate(sizes):
+        h = dev.alloc(2 * s)
+        assert dev.lib.gm_fill_normal_f16(dev.handle, h, s, seed + k, 0.0, std, scale) == 0
+        handles.append(h)
+        host.append(dev.to_numpy(h, s, np.uint16))
+    return handles, host
+
+
+def poke_half(dev, handle, index, bits):
+    """Overwrites one fp16 element of a device buffer (2-byte device-to-device copy)."""
+    tmp = dev.from_numpy(np.array([bits, 0], np.uint16))
+    assert dev.lib.copy_buffer_to_buffer_sync(tmp, handle, 0, 2 * index, 2) == 0
+    dev.free(tmp)
+
+
+@pytest.mark.parametrize("name,sizes_fn,weight_decay", [
+    ("config4_125m", amp_125m_sizes, 0.0),
+    ("config5_1b", transformer_block_sizes, 1e-4),
+])
+def test_amp_full_size(dev, name, sizes_fn, weight_decay):
+    """Full-size tensor lists (125M / 60 tensors and 1.012B / 400 tensors): clean step, a step with
+    an injected -inf (every buffer must stay byte-identical), a step with a NaN, two clean steps;
+    then p / m / v / fp16 copy against the oracle, bit for bit."""
+    sizes = sizes_fn()
+    hyper = dict(HYPER, weight_decay=weight_decay)
+    rng = np.random.default_rng(17)
+    w = [rng.standard_normal(s, dtype=np.float32) * np.float32(0.02) for s in sizes]
+    pair = AmpPair(dev, w, hyper, nthreads=NTHREADS)
+    for h in pair.d["g16"]:
+        dev.free(h)
+    g_handles, g_host = device_normal_f16(dev, sizes, 0xABC, 1e-4, 65536.0)
+    pair.d["g16"] = g_handles
+    pair.c["g16"] = pair.pkg.handle_array(g_handles)
+    try:
+        assert pair.step(g_host, upload=False) == 0
+        victim = len(sizes) - 3
+        clean = int(g_host[victim][12345 % sizes[victim]])
+        for bits in (0xFC00, 0x7E00):
+            poke_half(dev, g_handles[victim], 12345 % sizes[victim], bits)
+            g_host[victim][12345 % sizes[victim]] = bits
+            assert pair.step(g_host, upload=False) == 1
+        pair.compare("after skipped steps")          # includes: nothing moved since the clean step
+        poke_half(dev, g_handles[victim], 12345 % sizes[victim], clean)
+        g_host[victim][12345 % sizes[victim]] = clean
+        assert pair.step(g_host, upload=False) == 0
+        assert pair.step(g_host, upload=False) == 0
+        assert float(np.float32(pair.st.scale)) == 16384.0 and pair.st.step_count == 3
+        pair.compare("final")
+    finally:
+        pair.close()

@@ -1,0 +1,147 @@
+"""Buffer primitives of the C ABI on the GPU.  The first three tests restate the reference's
+exact-equality device tests (cgo_bridge/bridge_test.go:188-276, advanced_test.go:53-98)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from harness import gpu_device
+from oracle_lib import oracle
+
+pytestmark = pytest.mark.gpu
+vp = ctypes.c_void_p
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = gpu_device()
+    if d is None:
+        pytest.fail("libgometal_hip.so is missing or no GPU is usable: GPU tests cannot run")
+    return d
+
+
+def test_float32_round_trip(dev):                      # bridge_test.go:188-229
+    data = (np.arange(64, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    buf = dev.alloc(256)
+    assert dev.lib.copy_float32_array_to_metal_buffer(buf, data.ctypes.data_as(vp), 64) == 0
+    out = np.empty(64, np.float32)
+    assert dev.lib.copy_metal_buffer_to_float32_array(buf, out.ctypes.data_as(vp), 64) == 0
+    assert np.array_equal(out.view(np.uint32), data.view(np.uint32))
+    dev.free(buf)
+
+
+def test_zero_buffer(dev):                             # bridge_test.go:232-276
+    data = np.arange(1, 33, dtype=np.float32)
+    buf = dev.alloc(128)
+    dev.upload(buf, data)
+    assert dev.lib.zero_metal_buffer(dev.handle, buf, 128) == 0
+    assert np.all(dev.to_numpy(buf, 32).view(np.uint32) == 0)
+    dev.free(buf)
+
+
+def test_buffer_to_buffer_sync_copy(dev):              # advanced_test.go:53-98
+    data = (np.arange(64, dtype=np.float32) * np.float32(0.5)).astype(np.float32)
+    src, dst = dev.alloc(256), dev.alloc(256)
+    dev.upload(src, data)
+    assert dev.lib.copy_buffer_to_buffer_sync(src, dst, 0, 0, 256) == 0
+    assert np.array_equal(dev.to_numpy(dst, 64), data)
+    # offsets, and the range checks of bridge_memory.m:523-537
+    assert dev.lib.copy_buffer_to_buffer_sync(src, dst, 16, 32, 64) == 0
+    got = dev.to_numpy(dst, 64)
+    assert np.array_equal(got[8:24], data[4:20]) and np.array_equal(got[:8], data[:8])
+    assert dev.lib.copy_buffer_to_buffer_sync(src, dst, 200, 0, 64) == -4
+    assert dev.lib.copy_buffer_to_buffer_sync(src, dst, 0, 200, 64) == -5
+    dev.free(src)
+    dev.free(dst)
+
+
+@pytest.mark.parametrize("n", [1, 3, 5, 7, 255, 4097])
+def test_odd_sizes_and_canaries(dev, n):
+    """Zeroing and copying n floats must not touch the floats around them."""
+    total = n + 64
+    canary = np.full(total, np.float32(-123.5))
+    buf = dev.alloc(4 * total)
+    dev.upload(buf, canary)
+    assert dev.lib.zero_metal_buffer(dev.handle, buf, 4 * n) == 0
+    got = dev.to_numpy(buf, total)
+    assert np.all(got[:n] == 0) and np.all(got[n:] == np.float32(-123.5))
+    dev.free(buf)
+
+
+def test_allocation_length_is_rounded_to_16(dev):      # bridge_memory.m:28
+    for size, want in [(1, 16), (16, 16), (17, 32), (1000, 1008)]:
+        h = dev.lib.allocate_metal_buffer(dev.handle, size, 1)
+        assert h != 0 and h % 256 == 0
+        assert dev.lib.gm_buffer_length(h) == want
+        dev.lib.deallocate_metal_buffer(h)
+        assert dev.lib.gm_buffer_length(h) == 0
+
+
+def test_large_buffer_round_trip(dev):
+    """A 2^28-byte buffer: copy helpers hold up beyond small test sizes."""
+    n = (1 << 28) // 4
+    rng = np.random.default_rng(3)
+    data = rng.standard_normal(n, dtype=np.float32)
+    buf = dev.alloc(4 * n)
+    dev.upload(buf, data)
+    assert np.array_equal(dev.to_numpy(buf, n), data)
+    dev.free(buf)
+
+
+def all_half_patterns():
+    return np.arange(65536, dtype=np.uint32).astype(np.uint16)
+
+
+def test_convert_f16_to_f32_exhaustive(dev):
+    """Every binary16 pattern: the device widening equals the oracle's (NaNs compared as NaN)."""
+    h = all_half_patterns()
+    src = dev.from_numpy(h)
+    dst = dev.alloc(4 * h.size)
+    shape = (ctypes.c_int * 1)(h.size)
+    assert dev.lib.convert_tensor_type(src, dst, shape, 1, 2, 0, dev.handle) == 0
+    got = dev.to_numpy(dst, h.size)
+    want = oracle().f16_to_f32(h)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    dev.free(src)
+    dev.free(dst)
+
+
+def test_convert_f32_to_f16_boundaries_and_random(dev):
+    """Round-to-nearest-even narrowing: every half value, the midpoints between neighbouring halves
+    (ties), values one ulp either side of them, the overflow edge, subnormals, and random floats."""
+    o = oracle()
+    halves = o.f16_to_f32(all_half_patterns())
+    finite = np.sort(halves[np.isfinite(halves)].astype(np.float64))
+    mids = ((finite[:-1] + finite[1:]) / 2).astype(np.float32)
+    cases = [halves[np.isfinite(halves)], mids, np.nextafter(mids, np.float32(np.inf)),
+             np.nextafter(mids, np.float32(-np.inf)),
+             np.array([65504.0, 65519.99, 65520.0, 65536.0, 1e10, -65520.0, np.inf, -np.inf,
+                       5.9604645e-8, 2.9802322e-8, 2.9802325e-8, 1e-10, 0.0, -0.0, 1.0e-40], np.float32),
+             np.random.default_rng(11).standard_normal(200000).astype(np.float32) *
+             np.float32(10.0) ** np.random.default_rng(12).integers(-9, 6, 200000).astype(np.float32)]
+    x = np.concatenate(cases).astype(np.float32)
+    src = dev.from_numpy(x)
+    dst = dev.alloc(2 * x.size + 16)
+    shape = (ctypes.c_int * 2)(1, x.size)
+    assert dev.lib.convert_tensor_type(src, dst, shape, 2, 0, 2, dev.handle) == 0
+    got = dev.to_numpy(dst, x.size, np.uint16)
+    want = o.f32_to_f16(x)
+    assert np.array_equal(got, want)
+    # the unsupported pairs of the reference (bridge_memory.m:413-416)
+    assert dev.lib.convert_tensor_type(src, dst, shape, 2, 0, 0, dev.handle) == -3
+    dev.free(src)
+    dev.free(dst)
+
+
+def test_fill_normal_is_reproducible_and_sane(dev):
+    n = 1 << 20
+    a, b = dev.alloc(4 * n), dev.alloc(4 * n)
+    assert dev.lib.gm_fill_normal_f32(dev.handle, a, n, 42, 0.5, 2.0) == 0
+    assert dev.lib.gm_fill_normal_f32(dev.handle, b, n, 42, 0.5, 2.0) == 0
+    xa, xb = dev.to_numpy(a, n), dev.to_numpy(b, n)
+    assert np.array_equal(xa, xb)
+    assert abs(xa.mean() - 0.5) < 0.02 and abs(xa.std() - 2.0) < 0.02 and np.all(np.isfinite(xa))
+    dev.free(a)
+    dev.free(b)

@@ -1,0 +1,240 @@
+"""Properties of the CPU oracle that the mathematics fixes (closed forms, invariants, library
+casts): a dropped term, a wrong sign or a misplaced epsilon fails one of them."""
+import numpy as np
+import pytest
+
+from oracle_lib import oracle
+
+RNG = np.random.default_rng(2024)
+N = 4096
+
+
+def rand(scale, n=N):
+    return (RNG.standard_normal(n) * scale).astype(np.float32)
+
+
+def test_fp16_widening_matches_numpy_exhaustively():
+    h = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    got = oracle().f16_to_f32(h)
+    want = h.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_fp16_narrowing_matches_numpy():
+    o = oracle()
+    halves = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16).astype(np.float32)
+    finite = np.sort(halves[np.isfinite(halves)].astype(np.float64))
+    mids = ((finite[:-1] + finite[1:]) / 2).astype(np.float32)
+    x = np.concatenate([halves[np.isfinite(halves)], mids, np.nextafter(mids, np.float32(np.inf)),
+                        np.nextafter(mids, np.float32(-np.inf)),
+                        np.array([65504.0, 65519.99, 65520.0, 1e10, -1e10, np.inf, -np.inf, 0.0, -0.0,
+                                  5.9604645e-8, 2.9802322e-8, 2.9802325e-8, 1e-40], np.float32),
+                        rand(1.0, 100000) * np.float32(10.0) ** RNG.integers(-9, 6, 100000).astype(np.float32)])
+    x = x.astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(o.f32_to_f16(x), want)
+    nan = o.f32_to_f16(np.array([np.nan], np.float32)).view(np.float16)
+    assert np.isnan(nan[0])
+
+
+def test_adam_first_step_closed_form():
+    """t = 1, m = v = 0, wd = 0: m' = (1-b1) g, v' = (1-b2) g^2 and w' = w - lr * sign(g) for |g| >> eps."""
+    w, g = rand(0.02), rand(1e-2)
+    g[np.abs(g) < 1e-4] = np.float32(1e-3)
+    w0 = w.copy()
+    m, v = np.zeros(N, np.float32), np.zeros(N, np.float32)
+    oracle().adam(w, g, m, v, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1)
+    assert np.array_equal(m, g * (np.float32(1) - np.float32(0.9)))
+    assert np.array_equal(v, (g * g) * (np.float32(1) - np.float32(0.999)))
+    np.testing.assert_allclose(w0 - w, 1e-3 * np.sign(g), rtol=2e-4)
+
+
+def test_adam_against_float64_formula_and_decay_order():
+    """Ten steps against a float64 evaluation of the same formula; weight decay enters after the
+    adaptive term and before the lr multiply, on the pre-update weight."""
+    o = oracle()
+    # the hyper-parameters as the binary32 constants the host passes, evaluated in float64
+    lr, b1, b2, eps, wd = (float(np.float32(x)) for x in (1e-3, 0.9, 0.999, 1e-8, 1e-2))
+    w, m, v = rand(0.5), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    w64, m64, v64 = w.astype(np.float64), np.zeros(N), np.zeros(N)
+    for t in range(1, 11):
+        g = rand(1e-2)
+        o.adam(w, g, m, v, lr, b1, b2, eps, wd, t)
+        g64 = g.astype(np.float64)
+        m64 = b1 * m64 + (1 - b1) * g64
+        v64 = b2 * v64 + (1 - b2) * g64 * g64
+        upd = (m64 / (1 - b1 ** t)) / (np.sqrt(v64 / (1 - b2 ** t)) + eps) + wd * w64
+        w64 = w64 - lr * upd
+    np.testing.assert_allclose(w, w64, rtol=0, atol=2e-6)
+    np.testing.assert_allclose(m, m64, rtol=1e-5, atol=1e-9)
+    np.testing.assert_allclose(v, v64, rtol=1e-5, atol=1e-12)
+    # a decay applied to the gradient instead (the L2-into-grad variant) would differ visibly
+    w2, m2, v2 = rand(0.5), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    g = np.zeros(N, np.float32)
+    w2_0 = w2.copy()
+    o.adam(w2, g, m2, v2, lr, b1, b2, eps, wd, 1)
+    assert np.all(m2 == 0) and np.all(v2 == 0)                 # moments never see the decay
+    np.testing.assert_allclose(w2, w2_0 * (1 - lr * wd), rtol=1e-6)   # zero gradient: w moves only by decay
+
+
+def test_adam_wd_zero_matches_torch_loosely():
+    """With wd = 0 torch.optim.Adam has the same epsilon placement; rounding order differs."""
+    torch = pytest.importorskip("torch")
+    w, m, v = rand(0.5, 512), np.zeros(512, np.float32), np.zeros(512, np.float32)
+    p = torch.tensor(w.copy(), requires_grad=True)
+    opt = torch.optim.Adam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+    for t in range(1, 6):
+        g = rand(1e-2, 512)
+        oracle().adam(w, g, m, v, 1e-3, 0.9, 0.999, 1e-8, 0.0, t)
+        p.grad = torch.tensor(g)
+        opt.step()
+    np.testing.assert_allclose(w, p.detach().numpy(), rtol=1e-5, atol=1e-7)
+
+
+def test_sgd_closed_forms():
+    o = oracle()
+    w, g = rand(0.1), rand(1e-2)
+    w0 = w.copy()
+    o.sgd(w, g, None, 0.01, 0.0, 0.0, False)
+    assert np.array_equal(w, w0 - np.float32(0.01) * g)            # vanilla: w - lr g
+    # momentum: first step m = g, w = w - lr g; second step m = mu m + g
+    w, m = w0.copy(), np.zeros(N, np.float32)
+    o.sgd(w, g, m, 0.01, 0.9, 0.0, False)
+    assert np.array_equal(m, g) and np.array_equal(w, w0 - np.float32(0.01) * g)
+    o.sgd(w, g, m, 0.01, 0.9, 0.0, False)
+    assert np.array_equal(m, g * np.float32(0.9) + g)
+    # Nesterov: upd = lr (mu m' + g); L2 decay goes into the gradient before the momentum
+    w, m = w0.copy(), np.zeros(N, np.float32)
+    o.sgd(w, g, m, 0.01, 0.9, 0.1, True)
+    g2 = g + w0 * np.float32(0.1)
+    assert np.array_equal(m, g2)
+    assert np.array_equal(w, w0 - np.float32(0.01) * (np.float32(0.9) * g2 + g2))
+
+
+def test_adagrad_closed_form_and_monotone_state():
+    o = oracle()
+    w, g, s = rand(0.1), rand(1e-2), np.zeros(N, np.float32)
+    w0 = w.copy()
+    o.adagrad(w, g, s, 0.01, 1e-10, 0.0)
+    assert np.array_equal(s, g * g)
+    # first step: w - (lr / (|g| + eps)) g, with the quotient formed before the product
+    want = w0 - (np.float32(0.01) / (np.sqrt(g * g) + np.float32(1e-10))) * g
+    assert np.array_equal(w, want)
+    prev = s.copy()
+    for _ in range(5):
+        o.adagrad(w, rand(1e-2), s, 0.01, 1e-10, 0.0)
+        assert np.all(s >= prev)
+        prev = s.copy()
+
+
+def test_adadelta_first_step_closed_form():
+    o = oracle()
+    rho, eps = np.float32(0.9), np.float32(1e-6)
+    w, g, s, a = rand(0.1), rand(1e-2), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    w0 = w.copy()
+    o.adadelta(w, g, s, a, 0.9, 1e-6, 0.0)
+    s1 = (g * g) * (np.float32(1) - rho)
+    d = (np.sqrt(eps) / np.sqrt(s1 + eps)) * g
+    assert np.array_equal(s, s1)
+    assert np.array_equal(w, w0 - d)
+    assert np.array_equal(a, (d * d) * (np.float32(1) - rho))
+    assert np.all(a >= 0) and np.all(s >= 0)
+
+
+def test_rmsprop_epsilon_inside_the_root_and_variants():
+    o = oracle()
+    w, g, s = rand(0.1), rand(1e-2), np.zeros(N, np.float32)
+    w0 = w.copy()
+    o.rmsprop(w, g, s, None, None, 0.01, 0.99, 1e-8, 0.0, 0.0, False)
+    s1 = (g * g) * (np.float32(1) - np.float32(0.99))
+    assert np.array_equal(s, s1)
+    assert np.array_equal(w, w0 - (g / np.sqrt(s1 + np.float32(1e-8))) * np.float32(0.01))
+    # zero gradient: the root is sqrt(eps), never a division by zero
+    wz, sz = w0.copy(), np.zeros(N, np.float32)
+    o.rmsprop(wz, np.zeros(N, np.float32), sz, None, None, 0.01, 0.99, 1e-8, 0.0, 0.0, False)
+    assert np.array_equal(wz, w0)
+    # momentum and centered states are persisted
+    w, s, b, ga = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    o.rmsprop(w, g, s, b, ga, 0.01, 0.99, 1e-8, 0.0, 0.9, True)
+    ga1 = g * (np.float32(1) - np.float32(0.99))
+    assert np.array_equal(ga, ga1)
+    u = g / np.sqrt((s1 - ga1 * ga1) + np.float32(1e-8))
+    assert np.array_equal(b, u) and np.array_equal(w, w0 - u * np.float32(0.01))
+
+
+def test_nadam_against_float64_formula():
+    o = oracle()
+    lr, b1, b2, eps = (float(np.float32(x)) for x in (0.002, 0.9, 0.999, 1e-8))
+    w, m, v = rand(0.5), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    w64, m64, v64 = w.astype(np.float64), np.zeros(N), np.zeros(N)
+    for t in range(1, 8):
+        g = rand(1e-2)
+        o.nadam(w, g, m, v, lr, b1, b2, eps, 0.0, t)
+        g64 = g.astype(np.float64)
+        mu = b1 * (1 - 0.5 * 0.96 ** ((t + 1) * 0.004))
+        m64 = b1 * m64 + (1 - b1) * g64
+        v64 = b2 * v64 + (1 - b2) * g64 * g64
+        bc1, bc2 = 1 - b1 ** t, 1 - b2 ** t
+        mbar = mu * m64 / bc1 + (1 - mu) * g64 / bc1
+        w64 = w64 - lr * mbar / (np.sqrt(v64 / bc2) + eps)
+    np.testing.assert_allclose(w, w64, rtol=0, atol=3e-6)
+
+
+def test_threaded_oracle_equals_scalar_oracle():
+    o = oracle()
+    n = 100003
+    w, g = rand(0.02, n), rand(1e-2, n)
+    a = [w.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)]
+    b = [w.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)]
+    for t in (1, 2, 3):
+        o.adam(a[0], g, a[1], a[2], 1e-3, 0.9, 0.999, 1e-8, 1e-4, t, nthreads=1)
+        o.adam(b[0], g, b[1], b[2], 1e-3, 0.9, 0.999, 1e-8, 1e-4, t, nthreads=8)
+    for x, y in zip(a, b):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+
+
+def amp_reference_sequence(flags, init_scale, growth, backoff, interval):
+    """Brute-force state machine in pure Python over a list of overflow flags."""
+    scale, tracker, steps, out = np.float32(init_scale), 0, 0, []
+    for f in flags:
+        if f:
+            scale, tracker = np.float32(scale * np.float32(backoff)), 0
+        else:
+            steps += 1
+            tracker += 1
+            if tracker == interval:
+                scale, tracker = np.float32(scale * np.float32(growth)), 0
+        out.append((int(f), float(scale), tracker, steps))
+    return out
+
+
+def test_amp_skip_and_scale_sequence_against_brute_force():
+    o = oracle()
+    rng = np.random.default_rng(7)
+    sizes = [33, 7, 128]
+    flags = rng.random(400) < 0.08
+    st = o.amp_state(65536.0, 2.0, 0.5, 5)
+    w = [rand(0.1, n) for n in sizes]
+    m = [np.zeros(n, np.float32) for n in sizes]
+    v = [np.zeros(n, np.float32) for n in sizes]
+    w16 = [np.zeros(n, np.uint16) for n in sizes]
+    want = amp_reference_sequence(flags, 65536.0, 2.0, 0.5, 5)
+    for k, f in enumerate(flags):
+        # clipped so that only the injected elements overflow (the scale itself grows without bound here)
+        g16 = [np.clip(rng.standard_normal(n) * 1e-4 * st.scale, -6e4, 6e4).astype(np.float16).view(np.uint16)
+               for n in sizes]
+        if f:
+            t = int(rng.integers(0, len(sizes)))
+            g16[t][int(rng.integers(0, sizes[t]))] = [0x7C00, 0xFC00, 0x7E00][k % 3]
+        before = [a.copy() for a in w + m + v] + [a.copy() for a in w16]
+        skipped = o.adam_amp(w, g16, m, v, w16, 1e-3, 0.9, 0.999, 1e-8, 0.0, st)
+        assert (skipped, float(np.float32(st.scale)), st.growth_tracker, st.step_count) == want[k], k
+        if skipped:                      # a skipped step leaves every buffer byte-identical
+            for x, y in zip(before, w + m + v + w16):
+                assert np.array_equal(x.view(np.uint8), y.view(np.uint8))
+        else:
+            for a, h in zip(w, w16):
+                assert np.array_equal(h, a.astype(np.float16).view(np.uint16))
