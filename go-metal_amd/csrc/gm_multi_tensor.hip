@@ -3,7 +3,7 @@
 // cgo_bridge/bridge_optimizer.m).
 //
 // One launch per step.  The parameter list is cut into chunks of
-// chunk_elements (default 16384) and each chunk into slices of 256 * VEC
+// chunk_elements (4096 to 65536, chosen per list) and each chunk into slices of 256 * VEC
 // elements; workgroup b handles slice (b mod slices_per_chunk) of chunk
 // (b div slices_per_chunk), one VEC-wide group per lane: load every stream
 // once, apply the rule in registers, store every state once, exit.
@@ -32,12 +32,13 @@ namespace gm {
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBlock = 256;
-constexpr int kDefaultChunkElements = 16384;
+constexpr int kAutoChunkCandidates[] = {65536, 16384, 4096};   // largest first
+constexpr double kAutoChunkMaxIdleFraction = 0.05;
 constexpr int kDefaultVec = 1;
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 constexpr size_t kMaxCachedPlans = 16;
 
-static std::atomic<int> g_chunk_elements{kDefaultChunkElements};
+static std::atomic<int> g_chunk_elements{0};   // 0: chosen per plan
 static std::atomic<int> g_nontemporal{1};
 static std::atomic<int> g_vec{kDefaultVec};
 
@@ -64,7 +65,7 @@ MultiTensorPlan::~MultiTensorPlan()
 static bool plan_matches(const MultiTensorPlan &p, const PlanRequest &r, int chunk, uint64_t gen)
 {
     if (p.kind != r.kind || p.variant != r.variant || p.num_tensors != r.num_tensors ||
-        p.chunk_elements != chunk || p.generation != gen)
+        p.requested_chunk_elements != chunk || p.generation != gen)
         return false;
     const size_t n = (size_t)r.num_tensors;
     if (n == 0) return true;
@@ -81,11 +82,35 @@ static bool plan_matches(const MultiTensorPlan &p, const PlanRequest &r, int chu
     return true;
 }
 
-static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanRequest &r, int chunk,
+// Chunk size for a tensor list when the caller has not fixed one.  A chunk's
+// descriptor is fetched once per workgroup, and that fetch is the only
+// latency a workgroup cannot overlap, so large chunks (many workgroups
+// sharing one cached descriptor) are faster; but every chunk launches a full
+// set of slices, and the slices past a tensor's end are idle workgroups.
+// Take the largest candidate whose idle workgroups stay below 5 % of the
+// working ones (lists of small tensors end up with small chunks).
+static int choose_chunk_elements(const PlanRequest &r)
+{
+    for (int candidate : kAutoChunkCandidates) {
+        const uint64_t per_chunk = (uint64_t)candidate / kBlock;
+        uint64_t working = 0, launched = 0;
+        for (int i = 0; i < r.num_tensors; i++) {
+            const uint64_t numel = r.sizes[i] > 0 ? (uint64_t)r.sizes[i] / sizeof(float) : 0;
+            working += (numel + kBlock - 1) / kBlock;
+            launched += (numel + candidate - 1) / candidate * per_chunk;
+        }
+        if (launched - working <= (uint64_t)(kAutoChunkMaxIdleFraction * (double)working)) return candidate;
+    }
+    return kAutoChunkCandidates[sizeof(kAutoChunkCandidates) / sizeof(int) - 1];
+}
+
+static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanRequest &r, int requested_chunk,
                                                    uint64_t gen)
 {
     auto plan = std::make_unique<MultiTensorPlan>();
     const size_t n = (size_t)r.num_tensors;
+    const int chunk = requested_chunk > 0 ? requested_chunk : choose_chunk_elements(r);
+    plan->requested_chunk_elements = requested_chunk;
     plan->kind = r.kind;
     plan->variant = r.variant;
     plan->num_tensors = r.num_tensors;
@@ -577,12 +602,14 @@ float gm_nadam_mu_next(float beta1, int step_count)
 int gm_set_tuning(int chunk_elements, int nontemporal, int vec)
 {
     const int v = vec == 0 ? kDefaultVec : vec;
-    const int c = chunk_elements == 0 ? kDefaultChunkElements : chunk_elements;
+    const int c = chunk_elements;
     if (v != 1 && v != 2 && v != 4) return -1;
-    // a chunk is a power-of-two number of 256 * vec element slices
-    if (c < kBlock * v || c % (kBlock * v) != 0) return -1;
-    const int slices = c / (kBlock * v);
-    if ((slices & (slices - 1)) != 0) return -1;
+    if (c != 0) {
+        // a chunk is a power-of-two number of 256 * vec element slices
+        if (c < kBlock * v || c % (kBlock * v) != 0) return -1;
+        const int slices = c / (kBlock * v);
+        if ((slices & (slices - 1)) != 0) return -1;
+    }
     g_vec.store(v);
     g_chunk_elements.store(c);
     g_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));

@@ -10,7 +10,7 @@
 //
 // A descriptor is one 64-byte line, fetched by a single wave-uniform (scalar)
 // load that hits in cache for all but the first workgroup of the chunk
-// (64 bytes of table per 16384 elements, i.e. per >= 320 KB of streamed data).
+// (64 bytes of table per 4096..65536 elements).
 #pragma once
 
 #include "gm_context.hpp"
@@ -59,7 +59,8 @@ struct MultiTensorPlan {
     int kind = 0;
     int variant = 0;             // rule-specific bits that change validation (e.g. which optional states are on)
     int num_tensors = 0;
-    int chunk_elements = 0;
+    int requested_chunk_elements = 0;   // 0: chosen by the planner
+    int chunk_elements = 0;             // the size in force for this plan
     uint64_t generation = 0;
     std::vector<uintptr_t> handles;   // kNumSlots * num_tensors, slot-major
     std::vector<int> sizes;
@@ -92,7 +93,7 @@ struct PlanRequest {
 // the caller holds).  nullptr on a HIP failure (error already recorded).
 MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req);
 
-// Elements per chunk currently in force (tunable for sweeps).
+// Elements per chunk forced by the caller (tunable for sweeps); 0 = chosen per plan.
 int current_chunk_elements();
 // Whether streaming accesses carry the non-temporal hint.
 bool current_nontemporal();
