@@ -118,6 +118,10 @@ def main():
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
+    # launch-shape overrides (gm_set_tuning), for re-measuring the comparison in DESIGN.md; 0 / -1 = default
+    ap.add_argument("--chunk", type=int, default=0, help="elements per chunk")
+    ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4")
+    ap.add_argument("--nontemporal", type=int, default=-1, help="1 / 0: non-temporal hint on / off")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the optimizer step shards without communication, and this "
@@ -127,6 +131,8 @@ def main():
     pkg = load_package()
     dev = pkg.Device()                 # raises if the library is not built or no GPU is visible
     lib, D = dev.lib, dev.handle
+    if lib.gm_set_tuning(args.chunk, args.nontemporal, args.vec) != 0:
+        sys.exit("invalid --chunk / --vec combination (a chunk is a power-of-two multiple of 256 * vec elements)")
 
     desc, sizes_fn, rule, hyper, grad_std = WORKLOADS[args.workload]
     sizes = sizes_fn()
@@ -194,7 +200,9 @@ def main():
         "ms_per_step": wall_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": desc, "tensors": n, "params": params, "rule": rule, "hyper": hyper},
+        "config": {"workload": desc, "tensors": n, "params": params, "rule": rule, "hyper": hyper,
+                   "launch": {"chunk": args.chunk or "auto", "vec": args.vec or 1,
+                              "nontemporal": args.nontemporal != 0}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": f"multi_tensor_update_kernel<{rule}>", "bytes_per_param": bpp,
