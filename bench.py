@@ -34,7 +34,7 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
-MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8400e10}
+MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10}
 
 from workloads import amp_125m_sizes, cnn_sizes, ragged_sizes, transformer_block_sizes  # noqa: E402
 
