@@ -102,6 +102,20 @@ HOST_ABI = {
     "gmo_step_amp": (i, [u, up, up, i, ip]),
     "gmo_loss_scale": (f, [u]),
     "gmo_growth_tracker": (i, [u]),
+    "gmo_tensor_new": (u, [ip, i, i, i]),
+    "gmo_tensor_retain": (u, [u]),
+    "gmo_tensor_release": (None, [u]),
+    "gmo_tensor_free": (None, [u]),
+    "gmo_tensor_buffer": (u, [u]),
+    "gmo_tensor_size": (i, [u]),
+    "gmo_tensor_ref_count": (i, [u]),
+    "gmo_tensor_dtype": (i, [u]),
+    "gmo_tensor_convert_to": (u, [u, i]),
+    "gmo_tensor_copy_float32_data": (i, [u, vp, i]),
+    "gmo_tensor_to_float32_slice": (i, [u, vp, i]),
+    "gmo_tensor_copy_from": (i, [u, u]),
+    "gmo_calculate_size": (i, [ip, i, i]),
+    "gmo_execute_step_with_precomputed_gradients": (i, [u, up, i, up, i]),
     "gmo_extract_buffer_index": (i, [c_str]),
     "gmo_calculate_tensor_size": (i, [ip, i]),
 }

@@ -1,5 +1,6 @@
 // Flat C view of the host-side mirror (include/gometal_optimizer.h).
 #include "optimizer.hpp"
+#include "tensor.hpp"
 
 #include "../../include/gometal_optimizer.h"
 
@@ -385,6 +386,78 @@ int gmo_growth_tracker(uintptr_t opt)
 {
     auto *a = adam_of(opt);
     return a ? a->GrowthTracker : -1;
+}
+
+static memory::Tensor *T(uintptr_t h) { return reinterpret_cast<memory::Tensor *>(h); }
+
+uintptr_t gmo_tensor_new(const int *shape, int ndims, int dtype, int device_type)
+{
+    auto [t, err] = memory::Tensor::NewTensor(std::vector<int>(shape, shape + (ndims > 0 ? ndims : 0)),
+                                              (memory::DataType)dtype, (memory::DeviceType)device_type);
+    if (!err.empty()) {
+        fail(err);
+        return 0;
+    }
+    ok();
+    return reinterpret_cast<uintptr_t>(t);
+}
+
+uintptr_t gmo_tensor_retain(uintptr_t tensor) { return reinterpret_cast<uintptr_t>(T(tensor)->Retain()); }
+void gmo_tensor_release(uintptr_t tensor) { if (tensor) T(tensor)->Release(); }
+void gmo_tensor_free(uintptr_t tensor) { delete T(tensor); }
+uintptr_t gmo_tensor_buffer(uintptr_t tensor) { return reinterpret_cast<uintptr_t>(T(tensor)->MetalBuffer()); }
+int gmo_tensor_size(uintptr_t tensor) { return T(tensor)->Size(); }
+int gmo_tensor_ref_count(uintptr_t tensor) { return T(tensor)->RefCount(); }
+int gmo_tensor_dtype(uintptr_t tensor) { return (int)T(tensor)->DType(); }
+
+uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype)
+{
+    auto [t, err] = T(tensor)->ConvertTo((memory::DataType)dtype);
+    if (!err.empty()) {
+        fail(err);
+        return 0;
+    }
+    ok();
+    return reinterpret_cast<uintptr_t>(t);
+}
+
+int gmo_tensor_copy_float32_data(uintptr_t tensor, const float *data, int n)
+{
+    Error e = T(tensor)->CopyFloat32Data(std::vector<float>(data, data + (n > 0 ? n : 0)));
+    return e.empty() ? ok() : fail(e);
+}
+
+int gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity)
+{
+    auto [data, err] = T(tensor)->ToFloat32Slice();
+    if (!err.empty()) return fail(err);
+    if ((int)data.size() > capacity) return fail(Errorf("output holds %d elements, tensor has %d", capacity, (int)data.size()));
+    std::memcpy(out, data.data(), data.size() * sizeof(float));
+    ok();
+    return (int)data.size();
+}
+
+int gmo_tensor_copy_from(uintptr_t dst, uintptr_t src)
+{
+    Error e = T(dst)->CopyFrom(T(src));
+    return e.empty() ? ok() : fail(e);
+}
+
+int gmo_calculate_size(const int *shape, int ndims, int dtype)
+{
+    return memory::calculateSize(std::vector<int>(shape, shape + (ndims > 0 ? ndims : 0)), (memory::DataType)dtype);
+}
+
+int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *weight_tensors, int num_weights,
+                                                const uintptr_t *gradient_tensors, int num_gradients)
+{
+    std::vector<memory::Tensor *> w, g;
+    for (int k = 0; k < num_weights; k++) w.push_back(T(weight_tensors[k]));
+    for (int k = 0; k < num_gradients; k++) g.push_back(T(gradient_tensors[k]));
+    static const char *names[] = {"SGD", "Adam", "RMSProp", "AdaGrad", "AdaDelta", "Nadam"};
+    Handle *h = H(opt);
+    Error e = engine::ExecuteStepWithPrecomputedGradients(h ? h->opt.get() : nullptr, w, g, h ? names[h->kind] : "Adam");
+    return e.empty() ? ok() : fail(e);
 }
 
 int gmo_extract_buffer_index(const char *name) { return extractBufferIndex(name ? name : ""); }

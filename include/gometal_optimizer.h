@@ -82,6 +82,27 @@ int   gmo_step_amp(uintptr_t adam, const uintptr_t *gradient16_buffers, const ui
 float gmo_loss_scale(uintptr_t adam);
 int   gmo_growth_tracker(uintptr_t adam);
 
+/* ---- memory.Tensor (memory/tensor.go): reference-counted tensor over a pooled buffer.
+ * dtype codes: Float32 = 0, Int32 = 1, Float16 = 2, Int8 = 3 (tensor.go:10-17). ---- */
+uintptr_t gmo_tensor_new(const int *shape, int ndims, int dtype, int device_type);   /* NewTensor, tensor.go:41 */
+uintptr_t gmo_tensor_retain(uintptr_t tensor);                 /* Retain; 0 if already released */
+void      gmo_tensor_release(uintptr_t tensor);                /* Release, tensor.go:78 */
+void      gmo_tensor_free(uintptr_t tensor);                   /* destroys the released object */
+uintptr_t gmo_tensor_buffer(uintptr_t tensor);                 /* MetalBuffer */
+int       gmo_tensor_size(uintptr_t tensor);                   /* Size, bytes */
+int       gmo_tensor_ref_count(uintptr_t tensor);              /* RefCount */
+int       gmo_tensor_dtype(uintptr_t tensor);
+uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype);  /* ConvertTo, tensor.go:166; same handle retained if the type matches */
+int       gmo_tensor_copy_float32_data(uintptr_t tensor, const float *data, int n);   /* tensor.go:189 */
+int       gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity);    /* tensor.go:341; returns the element count */
+int       gmo_tensor_copy_from(uintptr_t dst, uintptr_t src);  /* CopyFrom, tensor.go:248 */
+int       gmo_calculate_size(const int *shape, int ndims, int dtype);                 /* tensor.go:137 */
+
+/* engine.ExecuteStepWithPrecomputedGradients (engine/training_engine.go:100-147) for any optimizer:
+ * tensors -> buffer handles -> SetWeightBuffers -> Step.  A 0 entry is a nil tensor. */
+int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *weight_tensors, int num_weights,
+                                                const uintptr_t *gradient_tensors, int num_gradients);
+
 /* helpers (interface.go:56-76, adam.go:142-148) */
 int gmo_extract_buffer_index(const char *name);
 int gmo_calculate_tensor_size(const int *dims, int ndims);

@@ -209,3 +209,28 @@ def test_optimizer_state_json_round_trip_is_exact():
     for v in vals:
         assert np.float32(float("%.9g" % float(v))) == v or (v == 0)
     assert not math.isnan(vals.sum())
+
+
+# ---- memory.Tensor helpers
+@pytest.mark.parametrize("shape,dtype,expected", [          # memory_test.go:94-122
+    ([], 0, 0), ([1], 0, 4), ([10], 0, 40), ([3, 4], 0, 48), ([2, 3, 4], 0, 96), ([10], 1, 40), ([10], 2, 20),
+    ([10], 3, 10), ([10], 99, -1)])
+def test_calculate_size(shape, dtype, expected):
+    assert lib.gmo_calculate_size(pkg.int_array(shape) if shape else None, len(shape), dtype) == expected
+
+
+def test_new_tensor_without_global_manager_or_gpu_fails_cleanly():
+    if lib.gmo_get_global_memory_manager() == 0:
+        assert lib.gmo_tensor_new(pkg.int_array([4]), 1, 0, 1) == 0
+        assert lib.gmo_last_error().decode().startswith("failed to allocate buffer: ")
+
+
+def test_precomputed_gradient_step_argument_errors(vanilla_sgd):   # engine/training_engine.go:108-124
+    one = pkg.handle_array([0])
+    assert lib.gmo_execute_step_with_precomputed_gradients(vanilla_sgd.handle, one, 1, one, 0) == -1
+    assert lib.gmo_last_error().decode() == "weight tensors (1) and gradient tensors (0) count mismatch"
+    two = pkg.handle_array([0, 0])
+    assert lib.gmo_execute_step_with_precomputed_gradients(vanilla_sgd.handle, two, 2, two, 2) == -1
+    assert lib.gmo_last_error().decode() == "weight tensor 0 is nil"
+    assert lib.gmo_execute_step_with_precomputed_gradients(0, two, 2, two, 2) == -1
+    assert lib.gmo_last_error().decode() == "Adam optimizer not initialized"
