@@ -94,6 +94,8 @@ HOST_ABI = {
     "gmo_cleanup": (None, [u]),
     "gmo_get_state_json": (vp, [u]),
     "gmo_load_state_json": (i, [u, c_str]),
+    "gmo_get_checkpoint_json": (vp, [u]),
+    "gmo_load_checkpoint_json": (i, [u, c_str]),
     "gmo_get_field": (f, [u, c_str]),
     "gmo_state_buffer": (u, [u, c_str, i]),
     "gmo_uses_pooling": (i, [u]),
@@ -282,6 +284,17 @@ class HostOptimizer:
 
     def LoadStateJSON(self, text):
         return self._err(self.lib.gmo_load_state_json(self.handle, text.encode()))
+
+    def GetCheckpointJSON(self):
+        p = self.lib.gmo_get_checkpoint_json(self.handle)
+        if not p:
+            return None, self.lib.gmo_last_error().decode()
+        text = ctypes.string_at(p).decode()
+        self.lib.gmo_free_string(p)
+        return text, None
+
+    def LoadCheckpointJSON(self, text):
+        return self._err(self.lib.gmo_load_checkpoint_json(self.handle, text.encode()))
 
     def field(self, name):
         return self.lib.gmo_get_field(self.handle, name.encode())

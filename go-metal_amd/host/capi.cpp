@@ -226,6 +226,28 @@ int gmo_load_state_json(uintptr_t opt, const char *json)
     return e.empty() ? ok() : fail(e);
 }
 
+char *gmo_get_checkpoint_json(uintptr_t opt)
+{
+    auto [state, err] = H(opt)->opt->GetState();
+    if (!err.empty() || !state) {
+        fail(err);
+        return nullptr;
+    }
+    ok();
+    std::string js = state->ToCheckpointJSON();
+    char *out = (char *)std::malloc(js.size() + 1);
+    if (out) std::memcpy(out, js.c_str(), js.size() + 1);
+    return out;
+}
+
+int gmo_load_checkpoint_json(uintptr_t opt, const char *json)
+{
+    auto [state, perr] = OptimizerState::FromCheckpointJSON(json ? json : "");
+    if (!perr.empty()) return fail(perr);
+    Error e = H(opt)->opt->LoadState(&state);
+    return e.empty() ? ok() : fail(e);
+}
+
 float gmo_get_field(uintptr_t opt, const char *name)
 {
     Handle *h = H(opt);

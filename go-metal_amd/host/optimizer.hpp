@@ -42,6 +42,14 @@ struct OptimizerState {
     // encoding/json shape: {"type":..,"parameters":{..},"state_data":[{"name","shape","data","state_type"}]}
     std::string ToJSON() const;
     static std::pair<OptimizerState, Error> FromJSON(const std::string &text);
+
+    // The reference stores this object under the key "optimizer_state" of its JSON checkpoint
+    // (checkpoints/checkpoint.go:38-52, written by saveJSON :133-157).  FromCheckpointJSON pulls
+    // it out of such a file's text (error if the checkpoint has none); ToCheckpointJSON writes a
+    // checkpoint document that carries only the optimizer state and the metadata block
+    // (framework "go-metal", version "1.0.0"), which the reference's loadJSON decodes.
+    static std::pair<OptimizerState, Error> FromCheckpointJSON(const std::string &text);
+    std::string ToCheckpointJSON() const;
 };
 
 // optimizer/interface.go:13-43

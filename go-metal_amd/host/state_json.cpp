@@ -217,6 +217,45 @@ struct Parser {
 
 }  // namespace
 
+std::string OptimizerState::ToCheckpointJSON() const
+{
+    // field order of checkpoints.Checkpoint (checkpoint.go:38-52); a nil model spec and weight
+    // list encode as null, the zero TrainingState as zeros
+    std::string out = "{\"model_spec\":null,\"weights\":null,\"training_state\":{\"epoch\":0,\"step\":0,"
+                      "\"learning_rate\":0,\"best_loss\":0,\"best_accuracy\":0,\"total_steps\":0},"
+                      "\"optimizer_state\":";
+    out += ToJSON();
+    out += ",\"metadata\":{\"version\":\"1.0.0\",\"framework\":\"go-metal\","
+           "\"created_at\":\"0001-01-01T00:00:00Z\"}}";
+    return out;
+}
+
+std::pair<OptimizerState, Error> OptimizerState::FromCheckpointJSON(const std::string &text)
+{
+    Parser ps{text.data(), text.data() + text.size(), ""};
+    if (!ps.expect('{')) return {OptimizerState{}, ps.err};
+    if (!ps.peek('}')) {
+        for (;;) {
+            std::string key;
+            if (!ps.string(key) || !ps.expect(':')) return {OptimizerState{}, ps.err};
+            ps.ws();
+            if (key == "optimizer_state") {
+                if (ps.literal("null")) break;
+                const char *begin = ps.p;
+                if (!ps.skip()) return {OptimizerState{}, ps.err};
+                return FromJSON(std::string(begin, ps.p));
+            }
+            if (!ps.skip()) return {OptimizerState{}, ps.err};
+            if (ps.peek(',')) {
+                ps.p++;
+                continue;
+            }
+            break;
+        }
+    }
+    return {OptimizerState{}, Errorf("checkpoint has no optimizer state")};
+}
+
 std::pair<OptimizerState, Error> OptimizerState::FromJSON(const std::string &text)
 {
     OptimizerState st;

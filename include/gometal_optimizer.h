@@ -64,6 +64,11 @@ void     gmo_cleanup(uintptr_t opt);
 char    *gmo_get_state_json(uintptr_t opt);
 /* LoadState(state) with state decoded from JSON (every number becomes a float64, as in Go). */
 int      gmo_load_state_json(uintptr_t opt, const char *json);
+/* The same through the reference's JSON checkpoint document (checkpoints/checkpoint.go:38-52):
+ * GetState() wrapped as {"model_spec", "weights", "training_state", "optimizer_state", "metadata"},
+ * and LoadState() from the "optimizer_state" member of such a document. */
+char    *gmo_get_checkpoint_json(uintptr_t opt);
+int      gmo_load_checkpoint_json(uintptr_t opt, const char *json);
 
 /* Field access for tests: hyper-parameter by Go field name ("LearningRate", "Beta1", ...; bools
  * as 0 / 1); NaN if the optimizer has no such field. */

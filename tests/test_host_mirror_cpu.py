@@ -234,3 +234,28 @@ def test_precomputed_gradient_step_argument_errors(vanilla_sgd):   # engine/trai
     assert lib.gmo_last_error().decode() == "weight tensor 0 is nil"
     assert lib.gmo_execute_step_with_precomputed_gradients(0, two, 2, two, 2) == -1
     assert lib.gmo_last_error().decode() == "Adam optimizer not initialized"
+
+
+def test_optimizer_state_inside_a_reference_checkpoint_document(vanilla_sgd):
+    """checkpoints/checkpoint.go:38-52: the optimizer state travels under "optimizer_state" of the
+    JSON checkpoint (pretty-printed by saveJSON, :146-147).  Reading one back and writing one."""
+    doc = json.dumps({
+        "model_spec": {"layers": [{"name": "fc1", "type": 0, "params": {"a": [1, {"b": "}"}]}}]},
+        "weights": [{"name": "fc1.weight", "shape": [2, 2], "data": [1.0, 2.0, 3.0, 4.0], "layer": "fc1", "type": "weight"}],
+        "training_state": {"epoch": 3, "step": 42, "learning_rate": 0.01, "best_loss": 0.5, "best_accuracy": 0.9,
+                           "total_steps": 42},
+        "optimizer_state": {"type": "SGD", "parameters": {"learning_rate": 0.25, "momentum": 0.0, "nesterov": False,
+                                                          "step_count": 42, "weight_decay": 0.125},
+                            "state_data": []},
+        "metadata": {"version": "1.0.0", "framework": "go-metal", "created_at": "2025-01-01T00:00:00Z"}}, indent=2)
+    assert vanilla_sgd.LoadCheckpointJSON(doc) is None
+    assert vanilla_sgd.field("LearningRate") == 0.25 and vanilla_sgd.field("WeightDecay") == 0.125
+    assert vanilla_sgd.GetStepCount() == 42
+    text, err = vanilla_sgd.GetCheckpointJSON()
+    assert err is None
+    out = json.loads(text)
+    assert list(out) == ["model_spec", "weights", "training_state", "optimizer_state", "metadata"]
+    assert out["optimizer_state"]["type"] == "SGD" and out["optimizer_state"]["parameters"]["step_count"] == 42
+    assert out["metadata"]["framework"] == "go-metal"
+    assert vanilla_sgd.LoadCheckpointJSON(json.dumps({"weights": [], "metadata": {}})) == "checkpoint has no optimizer state"
+    assert vanilla_sgd.LoadCheckpointJSON(json.dumps({"optimizer_state": None})) == "checkpoint has no optimizer state"
