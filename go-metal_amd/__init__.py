@@ -118,6 +118,12 @@ HOST_ABI = {
     "gmo_tensor_copy_from": (i, [u, u]),
     "gmo_calculate_size": (i, [ip, i, i]),
     "gmo_execute_step_with_precomputed_gradients": (i, [u, up, i, up, i]),
+    "gmo_scheduler_new": (u, [i, i, ctypes.c_double, ctypes.c_double, c_str]),
+    "gmo_scheduler_free": (None, [u]),
+    "gmo_scheduler_get_lr": (ctypes.c_double, [u, i, i, ctypes.c_double]),
+    "gmo_scheduler_plateau_step": (ctypes.c_double, [u, ctypes.c_double, ctypes.c_double]),
+    "gmo_scheduler_name": (c_str, [u]),
+    "gmo_scheduler_apply": (ctypes.c_double, [u, u, i, i, ctypes.c_double]),
     "gmo_extract_buffer_index": (i, [c_str]),
     "gmo_calculate_tensor_size": (i, [ip, i]),
 }

@@ -1,5 +1,6 @@
 // Flat C view of the host-side mirror (include/gometal_optimizer.h).
 #include "optimizer.hpp"
+#include "scheduler.hpp"
 #include "tensor.hpp"
 
 #include "../../include/gometal_optimizer.h"
@@ -480,6 +481,50 @@ int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *
     Handle *h = H(opt);
     Error e = engine::ExecuteStepWithPrecomputedGradients(h ? h->opt.get() : nullptr, w, g, h ? names[h->kind] : "Adam");
     return e.empty() ? ok() : fail(e);
+}
+
+struct SchedulerHandle {
+    int kind;
+    std::unique_ptr<training::LRScheduler> s;
+    std::string name;
+};
+
+uintptr_t gmo_scheduler_new(int kind, int a, double b, double c, const char *mode)
+{
+    auto *h = new SchedulerHandle{kind, nullptr, ""};
+    switch (kind) {
+    case 0: h->s = std::make_unique<training::StepLRScheduler>(a, b); break;
+    case 1: h->s = std::make_unique<training::ExponentialLRScheduler>(b); break;
+    case 2: h->s = std::make_unique<training::CosineAnnealingLRScheduler>(a, b); break;
+    case 3: h->s = std::make_unique<training::ReduceLROnPlateauScheduler>(b, a, c, mode ? mode : ""); break;
+    case 4: h->s = std::make_unique<training::NoOpScheduler>(); break;
+    default: delete h; fail(Errorf("unknown scheduler kind %d", kind)); return 0;
+    }
+    h->name = h->s->GetName();
+    return reinterpret_cast<uintptr_t>(h);
+}
+
+void gmo_scheduler_free(uintptr_t scheduler) { delete reinterpret_cast<SchedulerHandle *>(scheduler); }
+
+double gmo_scheduler_get_lr(uintptr_t scheduler, int epoch, int step, double base_lr)
+{
+    return reinterpret_cast<SchedulerHandle *>(scheduler)->s->GetLR(epoch, step, base_lr);
+}
+
+double gmo_scheduler_plateau_step(uintptr_t scheduler, double metric, double current_lr)
+{
+    auto *h = reinterpret_cast<SchedulerHandle *>(scheduler);
+    if (h->kind != 3) return std::nan("");
+    return static_cast<training::ReduceLROnPlateauScheduler *>(h->s.get())->Step(metric, current_lr);
+}
+
+const char *gmo_scheduler_name(uintptr_t scheduler) { return reinterpret_cast<SchedulerHandle *>(scheduler)->name.c_str(); }
+
+double gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, int step, double base_lr)
+{
+    const double lr = gmo_scheduler_get_lr(scheduler, epoch, step, base_lr);
+    H(opt)->opt->UpdateLearningRate((float)lr);
+    return lr;
 }
 
 int gmo_extract_buffer_index(const char *name) { return extractBufferIndex(name ? name : ""); }

@@ -108,6 +108,18 @@ int       gmo_calculate_size(const int *shape, int ndims, int dtype);           
 int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *weight_tensors, int num_weights,
                                                 const uintptr_t *gradient_tensors, int num_gradients);
 
+/* ---- learning-rate schedules (training/scheduler.go).  kind: 0 StepLR(a = stepSize, b = gamma),
+ * 1 ExponentialLR(b = gamma), 2 CosineAnnealingLR(a = tMax, b = etaMin),
+ * 3 ReduceLROnPlateau(a = patience, b = factor, c = threshold, mode "min" / "max"), 4 constant. ---- */
+uintptr_t   gmo_scheduler_new(int kind, int a, double b, double c, const char *mode);
+void        gmo_scheduler_free(uintptr_t scheduler);
+double      gmo_scheduler_get_lr(uintptr_t scheduler, int epoch, int step, double base_lr);   /* GetLR */
+double      gmo_scheduler_plateau_step(uintptr_t scheduler, double metric, double current_lr);/* Step (kind 3 only; else NaN) */
+const char *gmo_scheduler_name(uintptr_t scheduler);                                          /* GetName */
+/* GetLR followed by the optimizer's UpdateLearningRate(float32(lr)), the fan-out of
+ * engine/model_engine.go:2332-2390.  Returns the rate that was set. */
+double      gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, int step, double base_lr);
+
 /* helpers (interface.go:56-76, adam.go:142-148) */
 int gmo_extract_buffer_index(const char *name);
 int gmo_calculate_tensor_size(const int *dims, int ndims);

@@ -259,3 +259,34 @@ def test_optimizer_state_inside_a_reference_checkpoint_document(vanilla_sgd):
     assert out["metadata"]["framework"] == "go-metal"
     assert vanilla_sgd.LoadCheckpointJSON(json.dumps({"weights": [], "metadata": {}})) == "checkpoint has no optimizer state"
     assert vanilla_sgd.LoadCheckpointJSON(json.dumps({"optimizer_state": None})) == "checkpoint has no optimizer state"
+
+
+# ---- learning-rate schedules (training/scheduler.go)
+def test_lr_schedulers_follow_the_reference_formulas(vanilla_sgd):
+    mk = lib.gmo_scheduler_new
+    step = mk(0, 30, 0.1, 0.0, None)
+    assert lib.gmo_scheduler_name(step) == b"StepLR"
+    assert [lib.gmo_scheduler_get_lr(step, e, 0, 0.1) for e in (0, 29, 30, 65)] == \
+        [0.1, 0.1, 0.1 * math.pow(0.1, 1.0), 0.1 * math.pow(0.1, 2.0)]
+    bad = mk(0, -5, 7.0, 0.0, None)                       # invalid arguments fall back to 30 / 0.1 (scheduler.go:26-31)
+    assert lib.gmo_scheduler_get_lr(bad, 30, 0, 1.0) == 0.1
+    expo = mk(1, 0, 0.95, 0.0, None)
+    assert lib.gmo_scheduler_get_lr(expo, 10, 0, 0.01) == 0.01 * math.pow(0.95, 10.0)
+    cos = mk(2, 100, 1e-5, 0.0, None)
+    assert lib.gmo_scheduler_get_lr(cos, 0, 0, 0.1) == 0.1
+    assert lib.gmo_scheduler_get_lr(cos, 50, 0, 0.1) == 1e-5 + (0.1 - 1e-5) * (1 + math.cos(math.pi * 50 / 100)) / 2
+    assert lib.gmo_scheduler_get_lr(cos, 100, 0, 0.1) == 1e-5 and lib.gmo_scheduler_get_lr(cos, 500, 0, 0.1) == 1e-5
+    plateau = mk(3, 2, 0.5, 1e-4, b"min")
+    assert lib.gmo_scheduler_name(plateau) == b"ReduceLROnPlateau"
+    assert lib.gmo_scheduler_get_lr(plateau, 0, 0, 0.1) == 0.1          # not initialised yet: base LR
+    seq = [lib.gmo_scheduler_plateau_step(plateau, m, 0.1) for m in (1.0, 0.9, 0.95, 0.95, 0.95, 0.5, 0.6, 0.6)]
+    assert seq == [0.1, 0.1, 0.1, 0.05, 0.05, 0.05, 0.05, 0.025]
+    assert lib.gmo_scheduler_get_lr(plateau, 9, 0, 0.1) == 0.025
+    const = mk(4, 0, 0.0, 0.0, None)
+    assert lib.gmo_scheduler_name(const) == b"ConstantLR" and lib.gmo_scheduler_get_lr(const, 7, 3, 0.3) == 0.3
+    assert math.isnan(lib.gmo_scheduler_plateau_step(const, 1.0, 0.1))
+    # fan-out to the optimizer (engine/model_engine.go:2332-2390): the float32 of the scheduled rate
+    assert lib.gmo_scheduler_apply(expo, vanilla_sgd.handle, 3, 0, 0.01) == 0.01 * math.pow(0.95, 3.0)
+    assert vanilla_sgd.field("LearningRate") == f32(0.01 * math.pow(0.95, 3.0))
+    for h in (step, bad, expo, cos, plateau, const):
+        lib.gmo_scheduler_free(h)
