@@ -118,7 +118,7 @@ def main():
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
-    # launch-shape overrides (gm_set_tuning), for re-measuring the comparison in DESIGN.md; 0 / -1 = default
+    # launch-shape overrides (gm_set_tuning) for comparing lane widths and chunk sizes; 0 / -1 = default
     ap.add_argument("--chunk", type=int, default=0, help="elements per chunk")
     ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4")
     ap.add_argument("--nontemporal", type=int, default=-1, help="1 / 0: non-temporal hint on / off")

@@ -454,7 +454,7 @@ def main():
                           dict(lr=0.001, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0001),
                           w, [g] * 5, 5))
 
-    # BASELINE-config hyper-parameters, mixed signs and magnitudes, fresh gradient per step
+    # the benchmark configurations' hyper-parameters, mixed signs and magnitudes, fresh gradient per step
     n = 24
     wr = [rand_f32(rng, -8, 1) for _ in range(n)]
 
