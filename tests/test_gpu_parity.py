@@ -136,3 +136,37 @@ def test_variants_and_ragged_edges(dev, rule, hyper):
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
     run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
              steps=6, check_every=3, nthreads=1)
+
+
+SPECIALS = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-40, -3e-39, 1.17549435e-38,
+                     3.4028235e38, -3.4028235e38, 1e-30, 1e30, 1.0, -1.0, 65504.0, 1e-8, 5e-324], dtype=np.float32)
+
+
+@pytest.mark.parametrize("rule,hyper", [
+    ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=1e-4, nesterov=True)),
+    ("adam", dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)),
+    ("rmsprop", dict(lr=0.01, alpha=0.99, eps=1e-8, weight_decay=0.0, momentum=0.9, centered=True)),
+    ("adagrad", dict(lr=0.01, eps=1e-10, weight_decay=0.0)),
+    ("adadelta", dict(rho=0.9, eps=1e-6, weight_decay=0.0)),
+    ("nadam", dict(lr=0.002, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)),
+])
+def test_special_values(dev, rule, hyper):
+    """Every pairing of special weights and gradients (signed zeros, infinities, NaN, subnormals,
+    the largest finite value): the GPU and the oracle agree on where NaNs appear and on every other
+    bit -- subnormals are neither flushed on input nor on output, overflow goes to the same infinity."""
+    w = np.repeat(SPECIALS, SPECIALS.size).astype(np.float32)
+    g = np.tile(SPECIALS, SPECIALS.size).astype(np.float32)
+    gpu, cpu = GpuRun(dev, rule, hyper, [w]), OracleRun(rule, hyper, [w])
+    try:
+        with np.errstate(all="ignore"):
+            for _ in range(3):
+                gpu.step([g])
+                cpu.step([g])
+        got, want = gpu.snapshot(), cpu.snapshot()
+        for key in want:
+            a, b = got[key][0], want[key][0]
+            assert np.array_equal(np.isnan(a), np.isnan(b)), (rule, key, "NaN positions")
+            ok = ~np.isnan(b)
+            assert np.array_equal(a[ok].view(np.uint32), b[ok].view(np.uint32)), (rule, key)
+    finally:
+        gpu.close()
