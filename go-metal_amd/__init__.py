@@ -49,6 +49,10 @@ ABI = {
     "execute_adadelta_step_mpsgraph": (i, [u, up, up, up, up, i, ip, f, f, f]),
     "execute_adadelta_step_mpsgraph_pooled": (i, [u, up, up, up, up, i, ip, f, f, f, u]),
     "execute_nadam_step_mpsgraph": (i, [u, up, up, up, up, i, ip, f, f, f, f, f, i]),
+    "execute_lbfgs_step_mpsgraph": (i, [u, up, up, up, up, up, up, up, u, i, ip, i, i, i, f, f, f, i, f, f, fp]),
+    "execute_lbfgs_step_mpsgraph_pooled": (i, [u, up, up, up, up, up, up, up, u, i, ip, i, i, i, f, f, f, i, f, f,
+                                               u, fp]),
+    "gm_lbfgs_dot": (i, [u, up, up, i, ip, fp]),
     "gm_synchronize": (i, [u]),
     "gm_last_error": (ctypes.c_char_p, []),
     "gm_buffer_length": (ctypes.c_size_t, [u]),

@@ -1,0 +1,727 @@
+// L-BFGS step for gfx950: the HIP counterpart of execute_lbfgs_step_mpsgraph
+// (cgo_bridge/bridge_optimizer.m:980-1321), which the reference runs as CPU
+// loops over unified-memory buffers.
+//
+// The step is a fixed sequence of streaming launches over the whole tensor list
+// on one stream.  Every element-wise statement of the reference is one fused
+// pass; every dot product is accumulated by the pass that produces its operand,
+// so a history pair costs two passes, not four:
+//
+//   prologue     gather rho[idx(j)], mark pairs with |rho| < 1e-10 invalid, alpha[j] = 0 for them
+//   init         q = -g                       (+ dot(s_j, q) for the newest valid pair)
+//   backward     q -= alpha_j y_j             (+ dot with the next operand)
+//   forward      r += (alpha_j - beta) s_j    (+ dot with the next operand)
+//   update       p = -r; x += a p; old_g = g; s_cur = a p
+//   curvature    y_prev = g - old_g; rho_prev from dot(s_prev, y_prev)
+//
+// Which pairs are valid is read back once per step (history_count flags), so
+// only the passes that do work are launched; with the history the reference's
+// own optimizer produces (every rho it writes is 0) a step is the update pass
+// and the curvature pass.
+//
+// Dot products: exact fp64 products, summed in fp64 by a fixed radix-1024 tree
+// (lane l of a 256-lane workgroup adds elements l, l+256, l+512, l+768 of a
+// 1024-element slice in that order; lanes are combined by an adjacent-pair
+// binary tree; slice sums are reduced by the same node, 1024 at a time, until
+// one value is left) and rounded once to fp32.  The order is fixed by the data
+// layout alone, so results are bit-reproducible and independent of the launch
+// geometry.  The reference's running fp32 sum is inherently serial; this tree
+// lies within that sum's own rounding-error bound of it.
+#include "gm_context.hpp"
+
+#include "../../include/gometal_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <vector>
+
+namespace gm {
+
+bool current_nontemporal();   // gm_multi_tensor.hip
+
+namespace {
+
+constexpr int kLanes = 256;
+constexpr int kPerLane = 4;
+constexpr int kSlice = kLanes * kPerLane;            // 1024: the tree's radix and the slice length
+constexpr int kChunkCandidates[] = {65536, 16384, 4096, 1024};
+constexpr double kMaxIdleFraction = 0.05;
+
+struct alignas(16) LbChunk {
+    uint32_t tensor;        // index into the handle rows
+    uint32_t count;         // elements in this chunk
+    uint32_t offset;        // first element, relative to the tensor
+    uint32_t first_slice;   // ordinal of the chunk's first slice in the list-wide slice numbering
+};
+
+struct LbScalars {
+    float coef;             // coefficient of the next axpy pass, written by a reduction epilogue
+    float dot;              // last dot product, rounded to fp32
+};
+
+enum : int { kOpNone = 0, kOpAlpha, kOpBeta, kOpRho, kOpStore };
+
+struct Epilogue {
+    int op;
+    const float *rho;       // rho of the pair (kOpAlpha, kOpBeta)
+    float *alpha;           // &alpha[j] (kOpAlpha writes, kOpBeta reads)
+    float *rho_out;         // kOpRho
+    LbScalars *scalars;
+};
+
+struct Plan {
+    // key
+    std::vector<int> sizes;
+    uint64_t generation = 0;
+    // geometry
+    LbChunk *d_chunks = nullptr;
+    uint32_t num_chunks = 0;
+    uint32_t slice_shift = 0;          // log2(slices per chunk)
+    uint64_t total_slices = 0;
+    // handle rows: weights, gradients, old gradients, direction, s[h], y[h] (n each), then rho[h]
+    int history_size = 0;
+    std::vector<uintptr_t> handles;
+    uintptr_t alpha_handle = 0;
+    uintptr_t *d_handles = nullptr;
+    size_t handles_capacity = 0;
+    bool handles_valid = false;
+    // scratch
+    double *d_partial[2] = {nullptr, nullptr};
+    LbScalars *d_scalars = nullptr;
+    int *d_valid = nullptr;
+    int *h_valid = nullptr;            // pinned
+    int valid_capacity = 0;
+
+    ~Plan()
+    {
+        if (d_chunks) (void)hipFree(d_chunks);
+        if (d_handles) (void)hipFree(d_handles);
+        if (d_partial[0]) (void)hipFree(d_partial[0]);
+        if (d_partial[1]) (void)hipFree(d_partial[1]);
+        if (d_scalars) (void)hipFree(d_scalars);
+        if (d_valid) (void)hipFree(d_valid);
+        if (h_valid) (void)hipHostFree(h_valid);
+    }
+};
+
+constexpr size_t kMaxPlans = 4;
+// Never destroyed: plans own device memory, and static destructors may run after the HIP
+// runtime has shut down.
+std::vector<std::unique_ptr<Plan>> &plan_cache()
+{
+    static auto *cache = new std::vector<std::unique_ptr<Plan>>();
+    return *cache;
+}
+
+int choose_chunk(const int *sizes, int n)
+{
+    for (int candidate : kChunkCandidates) {
+        const uint64_t per_chunk = (uint64_t)candidate / kSlice;
+        uint64_t working = 0, launched = 0;
+        for (int i = 0; i < n; i++) {
+            const uint64_t numel = sizes[i] > 0 ? (uint64_t)sizes[i] / sizeof(float) : 0;
+            working += (numel + kSlice - 1) / kSlice;
+            launched += (numel + candidate - 1) / candidate * per_chunk;
+        }
+        if (launched - working <= (uint64_t)(kMaxIdleFraction * (double)working)) return candidate;
+    }
+    return kSlice;
+}
+
+// ---------------------------------------------------------------- kernels ----
+#define GM_GLOBAL __attribute__((address_space(1)))
+
+template <bool NT>
+__device__ inline float ld(const float *p)
+{
+    const GM_GLOBAL float *gp = (const GM_GLOBAL float *)p;
+    if (NT) return __builtin_nontemporal_load(gp);
+    return *gp;
+}
+
+template <bool NT>
+__device__ inline void st(float v, float *p)
+{
+    GM_GLOBAL float *gp = (GM_GLOBAL float *)p;
+    if (NT) __builtin_nontemporal_store(v, gp);
+    else *gp = v;
+}
+
+// Adjacent-pair binary tree over the 256 lane values of a workgroup; the result is valid in
+// thread 0.  The xor butterfly gives every lane of a pair the same sum (IEEE addition is
+// commutative), so after the step with distance d every lane holds the sum of its aligned
+// group of 2d lanes: exactly the adjacent-pair tree.
+__device__ inline double workgroup_tree(double v)
+{
+    __shared__ double wave_sum[kLanes / 64];
+#pragma unroll
+    for (int d = 1; d < 64; d *= 2) v = v + __shfl_xor(v, d, 64);
+    if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+}
+
+enum : int { kModeInit = 0, kModeAxpy, kModeUpdate, kModeUpdateFromGrad, kModeCurvature, kModeDotOnly };
+
+struct StreamArgs {
+    const LbChunk *chunks;
+    uint32_t slice_shift;
+    // rows of the handle table (one device address per tensor); meaning depends on the mode
+    const uintptr_t *r0, *r1, *r2, *r3, *r4;
+    double *partial;               // slice sums (modes with a dot product)
+    const LbScalars *scalars;      // coefficient for kModeAxpy
+    float step;                    // kModeUpdate*
+    int subtract;                  // kModeAxpy: x - c v (backward loop) or x + c v (forward loop)
+};
+
+// One workgroup = one 1024-element slice: lane l handles elements l, l+256, l+512, l+768.
+//   kModeInit            r0 = g, r1 = direction, r2 = dot operand        q = -g
+//   kModeAxpy            r0 = direction, r1 = v, r2 = dot operand        x = x -/+ c v
+//   kModeUpdate          r0 = direction, r1 = w, r2 = g, r3 = old_g, r4 = s_cur
+//   kModeUpdateFromGrad  same, with r = -g formed in registers (no valid pair this step)
+//   kModeCurvature       r0 = g, r1 = old_g, r2 = s_prev, r3 = y_prev    y = g - old_g, dot(s, y)
+//   kModeDotOnly         r0 = a, r1 = b
+template <int MODE, bool DOT, bool NT>
+__global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
+{
+    const LbChunk ch = a.chunks[blockIdx.x >> a.slice_shift];
+    const uint32_t slice = blockIdx.x & ((1u << a.slice_shift) - 1u);
+    const uint32_t base = slice * kSlice;
+    if (base >= ch.count) return;                       // the whole workgroup leaves together
+    const uint32_t left = ch.count - base;
+    const size_t first = (size_t)ch.offset + base + threadIdx.x;
+
+    float *p0 = reinterpret_cast<float *>(a.r0[ch.tensor]) + first;
+    float *p1 = reinterpret_cast<float *>(a.r1[ch.tensor]) + first;
+    float *p2 = nullptr, *p3 = nullptr, *p4 = nullptr;
+    constexpr bool kFusedDot = DOT && (MODE == kModeInit || MODE == kModeAxpy);   // r2 = dot operand
+    if (kFusedDot || MODE == kModeUpdate || MODE == kModeUpdateFromGrad || MODE == kModeCurvature)
+        p2 = reinterpret_cast<float *>(a.r2[ch.tensor]) + first;
+    if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad || MODE == kModeCurvature)
+        p3 = reinterpret_cast<float *>(a.r3[ch.tensor]) + first;
+    if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad)
+        p4 = reinterpret_cast<float *>(a.r4[ch.tensor]) + first;
+
+    float coef = 0.0f;
+    if (MODE == kModeAxpy) coef = a.scalars->coef;
+
+    double acc = 0.0;
+#pragma unroll
+    for (int u = 0; u < kPerLane; u++) {
+        const uint32_t i = threadIdx.x + u * kLanes;
+        if (i >= left) continue;
+        const size_t o = (size_t)u * kLanes;
+        float x = 0.0f, d = 0.0f;
+        if (MODE == kModeInit) {
+            x = -ld<NT>(p0 + o);
+            st<NT>(x, p1 + o);
+            if (DOT) d = ld<NT>(p2 + o);
+        } else if (MODE == kModeAxpy) {
+            const float xv = ld<NT>(p0 + o);
+            const float v = ld<NT>(p1 + o);
+            if (DOT) d = ld<NT>(p2 + o);
+            const float cv = coef * v;
+            x = a.subtract ? xv - cv : xv + cv;
+            st<NT>(x, p0 + o);
+        } else if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad) {
+            const float g = ld<NT>(p2 + o);
+            const float r = MODE == kModeUpdate ? ld<NT>(p0 + o) : -g;
+            const float w = ld<NT>(p1 + o);
+            const float p = -r;
+            const float sp = a.step * p;
+            st<NT>(p, p0 + o);
+            st<NT>(w + sp, p1 + o);
+            st<NT>(g, p3 + o);
+            st<NT>(sp, p4 + o);
+        } else if (MODE == kModeCurvature) {
+            const float g = ld<NT>(p0 + o);
+            const float og = ld<NT>(p1 + o);
+            d = ld<NT>(p2 + o);
+            x = g - og;
+            st<NT>(x, p3 + o);
+        } else {   // kModeDotOnly
+            x = ld<NT>(p0 + o);
+            d = ld<NT>(p1 + o);
+        }
+        if (DOT) acc = acc + (double)d * (double)x;     // exact product, one fp64 rounding per addition
+    }
+    if (DOT) {
+        const double total = workgroup_tree(acc);
+        if (threadIdx.x == 0) a.partial[ch.first_slice + slice] = total;
+    }
+}
+
+__device__ inline void run_epilogue(const Epilogue &e, double total)
+{
+    const float d = (float)total;
+    e.scalars->dot = d;
+    if (e.op == kOpAlpha) {
+        const float v = d * *e.rho;          // alpha_j = rho_j (s_j . q)
+        *e.alpha = v;
+        e.scalars->coef = v;
+    } else if (e.op == kOpBeta) {
+        const float beta = d * *e.rho;       // beta = rho_j (y_j . r)
+        e.scalars->coef = *e.alpha - beta;
+    } else if (e.op == kOpRho) {
+        *e.rho_out = fabs((double)d) > 1e-10 ? 1.0f / d : 0.0f;
+    }
+}
+
+// One tree level: workgroup b reduces src[1024 b .. 1024 b + 1023] to dst[b].  The launch with
+// a single workgroup is the last one and runs the scalar epilogue.
+__global__ void __launch_bounds__(kLanes) lbfgs_reduce_kernel(const double *__restrict__ src, uint64_t count,
+                                                             double *__restrict__ dst, Epilogue e)
+{
+    const uint64_t base = (uint64_t)blockIdx.x * kSlice;
+    const uint64_t left = count - base;
+    double acc = 0.0;
+#pragma unroll
+    for (int u = 0; u < kPerLane; u++) {
+        const uint32_t i = threadIdx.x + u * kLanes;
+        if (i < left) acc = acc + src[base + i];
+    }
+    const double total = workgroup_tree(acc);
+    if (threadIdx.x != 0) return;
+    dst[blockIdx.x] = total;
+    if (gridDim.x == 1 && e.op != kOpNone) run_epilogue(e, total);
+}
+
+// A list with zero or one slice has no tree level to run: the epilogue takes the value as is.
+__global__ void lbfgs_epilogue_kernel(const double *src, uint64_t count, Epilogue e)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    run_epilogue(e, count == 0 ? 0.0 : src[0]);
+}
+
+// rho of pair j of the recursion (slot idx(j) of the ring), validity flags, alpha[j] = 0 for
+// invalid pairs (bridge_optimizer.m:1078-1081).
+__global__ void lbfgs_prologue_kernel(const uintptr_t *rho_handles, int history_size, int history_count,
+                                      int history_index, float *alpha, int *valid)
+{
+    for (int j = threadIdx.x; j < history_count; j += blockDim.x) {
+        const int idx = (history_index - history_count + j + history_size) % history_size;
+        const float rho = *reinterpret_cast<const float *>(rho_handles[idx]);
+        const int ok = !(fabs((double)rho) < 1e-10);
+        valid[j] = ok;
+        if (!ok) alpha[j] = 0.0f;
+    }
+}
+
+// ------------------------------------------------------------------- host ----
+struct Rows {
+    const uintptr_t *w, *g, *old_g, *dir, *rho;
+    const uintptr_t *s(int h, int n) const { return s0 + (size_t)h * n; }
+    const uintptr_t *y(int h, int n) const { return y0 + (size_t)h * n; }
+    const uintptr_t *s0, *y0;
+};
+
+Rows rows_of(const uintptr_t *base, int n, int m)
+{
+    Rows r;
+    r.w = base;
+    r.g = base + (size_t)n;
+    r.old_g = base + (size_t)2 * n;
+    r.dir = base + (size_t)3 * n;
+    r.s0 = base + (size_t)4 * n;
+    r.y0 = r.s0 + (size_t)m * n;
+    r.rho = r.y0 + (size_t)m * n;
+    return r;
+}
+
+bool ensure_geometry(Context *ctx, Plan &p, const int *sizes, int n)
+{
+    const int chunk = choose_chunk(sizes, n);
+    std::vector<LbChunk> chunks;
+    uint64_t slice = 0;
+    for (int i = 0; i < n; i++) {
+        const size_t numel = sizes[i] > 0 ? (size_t)sizes[i] / sizeof(float) : 0;
+        for (size_t off = 0; off < numel; off += (size_t)chunk) {
+            const size_t left = numel - off;
+            LbChunk c;
+            c.tensor = (uint32_t)i;
+            c.count = (uint32_t)(left < (size_t)chunk ? left : (size_t)chunk);
+            c.offset = (uint32_t)off;
+            c.first_slice = (uint32_t)slice;
+            slice += (c.count + kSlice - 1) / kSlice;
+            chunks.push_back(c);
+        }
+    }
+    p.slice_shift = 0;
+    while ((1u << p.slice_shift) < (uint32_t)(chunk / kSlice)) p.slice_shift++;
+    if (slice > 0xFFFFFFFFull || ((uint64_t)chunks.size() << p.slice_shift) > 0x7FFFFFFFull) {
+        set_error("tensor list too large for one launch");
+        return false;
+    }
+    p.total_slices = slice;
+    p.num_chunks = (uint32_t)chunks.size();
+    p.sizes.assign(sizes, sizes + n);
+    if (!chunks.empty()) {
+        if (!hip_ok(hipMalloc(&p.d_chunks, chunks.size() * sizeof(LbChunk)), "hipMalloc(lbfgs chunks)") ||
+            !hip_ok(hipMemcpyAsync(p.d_chunks, chunks.data(), chunks.size() * sizeof(LbChunk),
+                                   hipMemcpyHostToDevice, ctx->stream), "upload lbfgs chunks") ||
+            !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+            return false;
+    }
+    const size_t level0 = (size_t)std::max<uint64_t>(slice, 1);
+    const size_t level1 = (level0 + kSlice - 1) / kSlice;
+    return hip_ok(hipMalloc(&p.d_partial[0], level0 * sizeof(double)), "hipMalloc(lbfgs partial sums)") &&
+           hip_ok(hipMalloc(&p.d_partial[1], level1 * sizeof(double)), "hipMalloc(lbfgs partial sums)") &&
+           hip_ok(hipMalloc(&p.d_scalars, sizeof(LbScalars)), "hipMalloc(lbfgs scalars)") &&
+           hip_ok(hipMemsetAsync(p.d_scalars, 0, sizeof(LbScalars), ctx->stream), "clear lbfgs scalars");
+}
+
+Plan *find_plan(Context *ctx, const int *sizes, int n)
+{
+    auto &cache = plan_cache();
+    const uint64_t gen = registry_generation();
+    for (size_t i = 0; i < cache.size(); i++) {
+        Plan &p = *cache[i];
+        if ((int)p.sizes.size() == n && std::memcmp(p.sizes.data(), sizes, (size_t)n * sizeof(int)) == 0) {
+            if (p.generation != gen) {       // handles may have been freed and reissued: revalidate
+                p.handles_valid = false;
+                p.generation = gen;
+            }
+            if (i != 0) std::rotate(cache.begin(), cache.begin() + i, cache.begin() + i + 1);
+            return cache[0].get();
+        }
+    }
+    auto plan = std::make_unique<Plan>();
+    plan->generation = gen;
+    if (!ensure_geometry(ctx, *plan, sizes, n)) return nullptr;
+    if (cache.size() >= kMaxPlans) {
+        (void)hipStreamSynchronize(ctx->stream);    // an evicted plan's scratch may still be in use
+        cache.pop_back();
+    }
+    cache.insert(cache.begin(), std::move(plan));
+    return cache[0].get();
+}
+
+// Flattens the caller's handle arrays, validates them on change and uploads the table.
+// Returns 0 or the entry point's error code.
+int stage_handles(Context *ctx, Plan &p, int n, int m, const uintptr_t *w, const uintptr_t *g,
+                  const uintptr_t *old_g, const uintptr_t *dir, const uintptr_t *s, const uintptr_t *y,
+                  const uintptr_t *rho, uintptr_t alpha)
+{
+    const size_t total = (size_t)(4 + 2 * m) * n + (size_t)m;
+    std::vector<uintptr_t> flat(total);
+    Rows r = rows_of(flat.data(), n, m);
+    const size_t row = (size_t)n * sizeof(uintptr_t);
+    std::memcpy(const_cast<uintptr_t *>(r.w), w, row);
+    std::memcpy(const_cast<uintptr_t *>(r.g), g, row);
+    std::memcpy(const_cast<uintptr_t *>(r.old_g), old_g, row);
+    std::memcpy(const_cast<uintptr_t *>(r.dir), dir, row);
+    std::memcpy(const_cast<uintptr_t *>(r.s0), s, row * m);
+    std::memcpy(const_cast<uintptr_t *>(r.y0), y, row * m);
+    std::memcpy(const_cast<uintptr_t *>(r.rho), rho, (size_t)m * sizeof(uintptr_t));
+    if (p.handles_valid && p.history_size == m && p.alpha_handle == alpha && p.handles == flat) return 0;
+
+    for (int i = 0; i < n; i++) {
+        const size_t need = p.sizes[i] > 0 ? (size_t)p.sizes[i] / sizeof(float) * sizeof(float) : 0;
+        for (int k = 0; k < 4 + 2 * m; k++) {
+            const uintptr_t h = flat[(size_t)k * n + i];
+            if (h == 0) {
+                set_error("L-BFGS buffer handle is nil (array %d, tensor %d)", k, i);
+                return -8;
+            }
+            const size_t have = registry_length(h);
+            if (have != 0 && have < need) {
+                set_error("L-BFGS buffer shorter than its tensor (array %d, tensor %d)", k, i);
+                return -8;
+            }
+        }
+    }
+    for (int h = 0; h < m; h++) {
+        if (r.rho[h] == 0) {
+            set_error("L-BFGS rho buffer %d is nil", h);
+            return -8;
+        }
+    }
+    const size_t alpha_len = registry_length(alpha);
+    if (alpha == 0 || (alpha_len != 0 && alpha_len < (size_t)m * sizeof(float))) {
+        set_error("L-BFGS alpha buffer is nil or shorter than history_size floats");
+        return -8;
+    }
+
+    if (p.handles_capacity < total) {
+        if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize")) return -8;
+        if (p.d_handles) (void)hipFree(p.d_handles);
+        p.d_handles = nullptr;
+        p.handles_capacity = 0;
+        if (!hip_ok(hipMalloc(&p.d_handles, total * sizeof(uintptr_t)), "hipMalloc(lbfgs handles)")) return -8;
+        p.handles_capacity = total;
+    }
+    if (p.valid_capacity < m) {
+        if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize")) return -8;
+        if (p.d_valid) (void)hipFree(p.d_valid);
+        if (p.h_valid) (void)hipHostFree(p.h_valid);
+        p.d_valid = nullptr;
+        p.h_valid = nullptr;
+        p.valid_capacity = 0;
+        if (!hip_ok(hipMalloc(&p.d_valid, (size_t)m * sizeof(int)), "hipMalloc(lbfgs flags)") ||
+            !hip_ok(hipHostMalloc(&p.h_valid, (size_t)m * sizeof(int), hipHostMallocDefault),
+                    "hipHostMalloc(lbfgs flags)"))
+            return -8;
+        p.valid_capacity = m;
+    }
+    // The staging vector dies with this call, so the upload is waited for.
+    if (!hip_ok(hipMemcpyAsync(p.d_handles, flat.data(), total * sizeof(uintptr_t), hipMemcpyHostToDevice,
+                               ctx->stream), "upload lbfgs handles") ||
+        !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+        return -8;
+    p.handles = std::move(flat);
+    p.history_size = m;
+    p.alpha_handle = alpha;
+    p.handles_valid = true;
+    return 0;
+}
+
+template <int MODE, bool DOT>
+void launch_stream(Context *ctx, const Plan &p, StreamArgs a)
+{
+    if (p.num_chunks == 0) return;
+    const uint32_t grid = p.num_chunks << p.slice_shift;
+    a.chunks = p.d_chunks;
+    a.slice_shift = p.slice_shift;
+    if (current_nontemporal()) lbfgs_stream_kernel<MODE, DOT, true><<<grid, kLanes, 0, ctx->stream>>>(a);
+    else lbfgs_stream_kernel<MODE, DOT, false><<<grid, kLanes, 0, ctx->stream>>>(a);
+}
+
+// Upper tree levels over the slice sums in d_partial[0], then the scalar epilogue.
+void launch_reduction(Context *ctx, const Plan &p, const Epilogue &e)
+{
+    uint64_t count = p.total_slices;
+    if (count <= 1) {
+        lbfgs_epilogue_kernel<<<1, 64, 0, ctx->stream>>>(p.d_partial[0], count, e);
+        return;
+    }
+    int src = 0;
+    const Epilogue none{kOpNone, nullptr, nullptr, nullptr, nullptr};
+    while (count > 1) {
+        const uint64_t next = (count + kSlice - 1) / kSlice;
+        lbfgs_reduce_kernel<<<(uint32_t)next, kLanes, 0, ctx->stream>>>(p.d_partial[src], count,
+                                                                        p.d_partial[src ^ 1],
+                                                                        next == 1 ? e : none);
+        count = next;
+        src ^= 1;
+    }
+}
+
+struct Entry {
+    Context *ctx = nullptr;
+    Plan *plan = nullptr;
+    std::unique_lock<std::mutex> lock;
+};
+
+int enter(uintptr_t device, const int *sizes, int n, Entry &out)
+{
+    clear_error();
+    if (device == 0) {
+        set_error("device handle is nil");
+        return -1;
+    }
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (n <= 0 || !sizes) {
+        set_error("L-BFGS needs at least one tensor and its size array");
+        return -8;
+    }
+    if (!make_current(ctx)) return -8;
+    out.lock = std::unique_lock<std::mutex>(ctx->mu);
+    out.ctx = ctx;
+    out.plan = find_plan(ctx, sizes, n);
+    return out.plan ? 0 : -8;
+}
+
+}  // namespace
+}  // namespace gm
+
+using namespace gm;
+
+extern "C" {
+
+int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uintptr_t *gradient_buffers,
+                                uintptr_t *old_gradient_buffers, uintptr_t *search_dir_buffers,
+                                uintptr_t *s_vectors_flat, uintptr_t *y_vectors_flat,
+                                uintptr_t *rho_buffers, uintptr_t alpha_buffer, int num_weights,
+                                int *buffer_sizes, int history_size, int history_count,
+                                int history_index, float initial_step, float c1, float c2,
+                                int max_line_search, float current_loss, float prev_loss,
+                                float *step_size)
+{
+    // The reference performs no line search: the Wolfe constants and the losses are accepted
+    // and ignored (bridge_optimizer.m:1231-1233).
+    (void)c1; (void)c2; (void)max_line_search; (void)current_loss; (void)prev_loss;
+    Entry en;
+    if (int rc = enter(device, buffer_sizes, num_weights, en)) return rc;
+    if (!weight_buffers || !gradient_buffers || !old_gradient_buffers || !search_dir_buffers ||
+        !s_vectors_flat || !y_vectors_flat || !rho_buffers) {
+        set_error("L-BFGS buffer arrays are required");
+        return -8;
+    }
+    if (history_size <= 0 || history_count < 0 || history_count > history_size || history_index < 0 ||
+        history_index >= history_size) {
+        set_error("L-BFGS history arguments out of range (size %d, count %d, index %d)", history_size,
+                  history_count, history_index);
+        return -5;
+    }
+    Context *ctx = en.ctx;
+    Plan &p = *en.plan;
+    const int n = num_weights, m = history_size;
+    if (int rc = stage_handles(ctx, p, n, m, weight_buffers, gradient_buffers, old_gradient_buffers,
+                               search_dir_buffers, s_vectors_flat, y_vectors_flat, rho_buffers, alpha_buffer))
+        return rc;
+    const Rows r = rows_of(p.d_handles, n, m);
+    const Rows host = rows_of(p.handles.data(), n, m);
+    float *alpha = reinterpret_cast<float *>(alpha_buffer);
+    hipStream_t stream = ctx->stream;
+    auto slot = [&](int j) { return (history_index - history_count + j + m) % m; };
+    auto rho_ptr = [&](int idx) { return reinterpret_cast<float *>(host.rho[idx]); };
+
+    // which pairs take part: one small read-back per step
+    std::vector<int> valid;
+    if (history_count > 0) {
+        lbfgs_prologue_kernel<<<1, 64, 0, stream>>>(r.rho, m, history_count, history_index, alpha, p.d_valid);
+        if (!hip_ok(hipGetLastError(), "L-BFGS prologue launch") ||
+            !hip_ok(hipMemcpyAsync(p.h_valid, p.d_valid, (size_t)history_count * sizeof(int),
+                                   hipMemcpyDeviceToHost, stream), "read L-BFGS pair flags") ||
+            !hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize"))
+            return -8;
+        for (int j = 0; j < history_count; j++)
+            if (p.h_valid[j]) valid.push_back(j);
+    }
+
+    StreamArgs base{};
+    base.partial = p.d_partial[0];
+    base.scalars = p.d_scalars;
+    base.step = initial_step;
+
+    if (valid.empty()) {
+        // q = -g, no recursion, p = -q: one pass
+        StreamArgs a = base;
+        a.r0 = r.dir; a.r1 = r.w; a.r2 = r.g; a.r3 = r.old_g; a.r4 = r.s(history_index, n);
+        launch_stream<kModeUpdateFromGrad, false>(ctx, p, a);
+    } else {
+        const int count = (int)valid.size();
+        // q = -g, with the first dot product of the backward loop
+        {
+            StreamArgs a = base;
+            a.r0 = r.g; a.r1 = r.dir; a.r2 = r.s(slot(valid[count - 1]), n);
+            launch_stream<kModeInit, true>(ctx, p, a);
+        }
+        // backward loop, newest pair first (bridge_optimizer.m:1046-1137)
+        for (int k = count - 1; k >= 0; k--) {
+            const int j = valid[k], idx = slot(j);
+            launch_reduction(ctx, p, Epilogue{kOpAlpha, rho_ptr(idx), alpha + j, nullptr, p.d_scalars});
+            StreamArgs a = base;
+            a.r0 = r.dir; a.r1 = r.y(idx, n); a.subtract = 1;
+            // next dot: s of the next older valid pair, or y of the oldest one (first forward dot)
+            a.r2 = k > 0 ? r.s(slot(valid[k - 1]), n) : r.y(slot(valid[0]), n);
+            launch_stream<kModeAxpy, true>(ctx, p, a);
+        }
+        // forward loop, oldest pair first (:1143-1216)
+        for (int k = 0; k < count; k++) {
+            const int j = valid[k], idx = slot(j);
+            launch_reduction(ctx, p, Epilogue{kOpBeta, rho_ptr(idx), alpha + j, nullptr, p.d_scalars});
+            StreamArgs a = base;
+            a.r0 = r.dir; a.r1 = r.s(idx, n); a.subtract = 0;
+            if (k + 1 < count) {
+                a.r2 = r.y(slot(valid[k + 1]), n);
+                launch_stream<kModeAxpy, true>(ctx, p, a);
+            } else {
+                launch_stream<kModeAxpy, false>(ctx, p, a);
+            }
+        }
+        // p = -r; x += a p; old_g = g; s_cur = a p  (:1219-1276)
+        StreamArgs a = base;
+        a.r0 = r.dir; a.r1 = r.w; a.r2 = r.g; a.r3 = r.old_g; a.r4 = r.s(history_index, n);
+        launch_stream<kModeUpdate, false>(ctx, p, a);
+    }
+    if (step_size) *step_size = initial_step;
+
+    // y_prev = g - old_g, rho_prev = 1 / (s_prev . y_prev)  (:1279-1335)
+    if (history_count > 0) {
+        const int prev = (history_index - 1 + m) % m;
+        StreamArgs a = base;
+        a.r0 = r.g; a.r1 = r.old_g; a.r2 = r.s(prev, n); a.r3 = r.y(prev, n);
+        launch_stream<kModeCurvature, true>(ctx, p, a);
+        launch_reduction(ctx, p, Epilogue{kOpRho, nullptr, nullptr, rho_ptr(prev), p.d_scalars});
+    }
+    return hip_ok(hipGetLastError(), "L-BFGS kernel launch") ? 0 : -8;
+}
+
+int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                       uintptr_t *gradient_buffers, uintptr_t *old_gradient_buffers,
+                                       uintptr_t *search_dir_buffers, uintptr_t *s_vectors_flat,
+                                       uintptr_t *y_vectors_flat, uintptr_t *rho_buffers,
+                                       uintptr_t alpha_buffer, int num_weights, int *buffer_sizes,
+                                       int history_size, int history_count, int history_index,
+                                       float initial_step, float c1, float c2, int max_line_search,
+                                       float current_loss, float prev_loss, uintptr_t command_pool,
+                                       float *step_size)
+{
+    // With or without a pool the reference runs the same code (bridge_optimizer.m:1365-1400).
+    (void)command_pool;
+    return execute_lbfgs_step_mpsgraph(device, weight_buffers, gradient_buffers, old_gradient_buffers,
+                                       search_dir_buffers, s_vectors_flat, y_vectors_flat, rho_buffers,
+                                       alpha_buffer, num_weights, buffer_sizes, history_size,
+                                       history_count, history_index, initial_step, c1, c2,
+                                       max_line_search, current_loss, prev_loss, step_size);
+}
+
+int gm_lbfgs_dot(uintptr_t device, uintptr_t *a_buffers, uintptr_t *b_buffers, int num_tensors,
+                 int *buffer_sizes, float *result)
+{
+    Entry en;
+    if (int rc = enter(device, buffer_sizes, num_tensors, en)) return rc;
+    if (!a_buffers || !b_buffers || !result) {
+        set_error("gm_lbfgs_dot: buffer arrays and result pointer are required");
+        return -8;
+    }
+    Context *ctx = en.ctx;
+    Plan &p = *en.plan;
+    const int n = num_tensors;
+    for (int i = 0; i < n; i++) {
+        const size_t need = buffer_sizes[i] > 0 ? (size_t)buffer_sizes[i] / sizeof(float) * sizeof(float) : 0;
+        for (uintptr_t h : {a_buffers[i], b_buffers[i]}) {
+            const size_t have = registry_length(h);
+            if (h == 0 || (have != 0 && have < need)) {
+                set_error("gm_lbfgs_dot: buffer %d is nil or shorter than its tensor", i);
+                return -8;
+            }
+        }
+    }
+    // a private two-row table; the step's cached table is left alone
+    uintptr_t *d_rows = nullptr;
+    LbScalars *h_result = nullptr;
+    std::vector<uintptr_t> rows((size_t)2 * n);
+    std::memcpy(rows.data(), a_buffers, (size_t)n * sizeof(uintptr_t));
+    std::memcpy(rows.data() + n, b_buffers, (size_t)n * sizeof(uintptr_t));
+    int rc = -8;
+    if (hip_ok(hipMalloc(&d_rows, rows.size() * sizeof(uintptr_t)), "hipMalloc(dot rows)") &&
+        hip_ok(hipHostMalloc(&h_result, sizeof(LbScalars), hipHostMallocDefault), "hipHostMalloc(dot result)") &&
+        hip_ok(hipMemcpyAsync(d_rows, rows.data(), rows.size() * sizeof(uintptr_t), hipMemcpyHostToDevice,
+                              ctx->stream), "upload dot rows")) {
+        StreamArgs a{};
+        a.partial = p.d_partial[0];
+        a.scalars = p.d_scalars;
+        a.r0 = d_rows;
+        a.r1 = d_rows + n;
+        launch_stream<kModeDotOnly, true>(ctx, p, a);
+        launch_reduction(ctx, p, Epilogue{kOpStore, nullptr, nullptr, nullptr, p.d_scalars});
+        if (hip_ok(hipGetLastError(), "dot kernel launch") &&
+            hip_ok(hipMemcpyAsync(h_result, p.d_scalars, sizeof(LbScalars), hipMemcpyDeviceToHost, ctx->stream),
+                   "read dot result") &&
+            hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize")) {
+            *result = h_result->dot;
+            rc = 0;
+        }
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (d_rows) (void)hipFree(d_rows);
+    if (h_result) (void)hipHostFree(h_result);
+    return rc;
+}
+
+}  // extern "C"

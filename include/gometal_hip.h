@@ -171,6 +171,42 @@ int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                 float learning_rate, float beta1, float beta2, float epsilon,
                                 float weight_decay, int step_count);
 
+/* bridge_optimizer.h:155-203 / .m:980-1404; prototypes bridge.go:296-343.  One L-BFGS step
+ * with the statement order of the reference's loop nest: q = -g; two-loop recursion over
+ * the history pairs whose |rho| >= 1e-10 (H0 = I); p = -r; x += initial_step * p (no line
+ * search: c1, c2, max_line_search and the losses are ignored, as in the reference);
+ * old_g = g; s[history_index] = initial_step * p; and, when history_count > 0,
+ * y[prev] = g - old_g and rho[prev] = 1 / (s[prev] . y[prev]) (0 when |s.y| <= 1e-10) for
+ * prev = history_index - 1.  s_vectors_flat / y_vectors_flat hold history_size * num_weights
+ * handles, entry [h * num_weights + i]; rho_buffers holds history_size handles of 4-byte
+ * buffers; alpha_buffer holds history_size floats.  *step_size = initial_step.
+ * Dot products are exact fp64 products summed by a fixed tree and rounded once to fp32
+ * (the reference keeps a running fp32 sum in element order).
+ * The call reads back which pairs are valid (it synchronises when history_count > 0); the
+ * passes themselves are asynchronous on the device's stream.
+ * -1 device 0; -3 no GPU; -5 history arguments out of range; -8 a handle or array is nil,
+ * a buffer of this library is shorter than its tensor, or a HIP error (the reference's
+ * exception code). */
+int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
+                                uintptr_t *gradient_buffers, uintptr_t *old_gradient_buffers,
+                                uintptr_t *search_dir_buffers, uintptr_t *s_vectors_flat,
+                                uintptr_t *y_vectors_flat, uintptr_t *rho_buffers,
+                                uintptr_t alpha_buffer, int num_weights, int *buffer_sizes,
+                                int history_size, int history_count, int history_index,
+                                float initial_step, float c1, float c2, int max_line_search,
+                                float current_loss, float prev_loss, float *step_size);
+/* bridge_optimizer.h:179-203 / .m:1338-1404: the same step (the pool is not used). */
+int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
+                                       uintptr_t *gradient_buffers,
+                                       uintptr_t *old_gradient_buffers,
+                                       uintptr_t *search_dir_buffers, uintptr_t *s_vectors_flat,
+                                       uintptr_t *y_vectors_flat, uintptr_t *rho_buffers,
+                                       uintptr_t alpha_buffer, int num_weights, int *buffer_sizes,
+                                       int history_size, int history_count, int history_index,
+                                       float initial_step, float c1, float c2,
+                                       int max_line_search, float current_loss, float prev_loss,
+                                       uintptr_t command_pool, float *step_size);
+
 /* ------------------------------------------------------------------------ */
 /* Additions (no counterpart in the reference's C ABI).                       */
 /* ------------------------------------------------------------------------ */
@@ -224,6 +260,11 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
                           float beta2, float epsilon, float weight_decay, int step_count,
                           uintptr_t amp_state, int *skipped, float *scale_out,
                           int *growth_tracker_out);
+
+/* The dot product of two tensor lists exactly as the L-BFGS step forms it (fp64 tree,
+ * one rounding to fp32).  Synchronises.  Codes as execute_lbfgs_step_mpsgraph. */
+int gm_lbfgs_dot(uintptr_t device, uintptr_t *a_buffers, uintptr_t *b_buffers, int num_tensors,
+                 int *buffer_sizes, float *result);
 
 /* Measurement helpers used by the benchmark and the profiles. */
 

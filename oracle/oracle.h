@@ -107,6 +107,25 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
                             float lr, float beta1, float beta2, float eps, float weight_decay,
                             gm_oracle_amp_state *st, int nthreads);
 
+/* L-BFGS step, cgo_bridge/bridge_optimizer.m:980-1321 (oracle_lbfgs.c states what is
+ * reproduced).  s and y hold history_size * num_tensors tensors, entry [h * num_tensors + i];
+ * rho and alpha are host arrays of history_size floats (the reference keeps each rho in a
+ * 4-byte buffer of its own).  Returns 0, or -5 for history arguments out of range.
+ *
+ * Pinning status: the reference's tests assert no numerical output of this function
+ * (optimizer/lbfgs_test.go checks construction, counters and error strings only).  The
+ * statement order is pinned by tests/golden/lbfgs_kat.json, written by an independent
+ * Python evaluator (numpy float32 element ops; Python floats for the fp64 tree), by the
+ * closed form w' = w + initial_step * g for an empty history, and, for GM_ORACLE_DOT_TREE,
+ * by agreement with the exactly rounded dot product (math.fsum) to 1 ulp. */
+enum { GM_ORACLE_DOT_REFERENCE = 0, GM_ORACLE_DOT_TREE = 1 };
+float gm_oracle_lbfgs_dot(const float *const *a, const float *const *b, const size_t *n, int num_tensors,
+                          int dot_mode, int per_tensor);
+int gm_oracle_lbfgs_step(float *const *w, const float *const *g, float *const *old_g, float *const *dir,
+                         float *const *s, float *const *y, float *rho, float *alpha,
+                         const size_t *n, int num_tensors, int history_size, int history_count,
+                         int history_index, float initial_step, int dot_mode, float *step_size);
+
 #ifdef __cplusplus
 }
 #endif

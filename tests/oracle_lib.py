@@ -55,6 +55,12 @@ class Oracle:
         for fn in (L.gm_oracle_sgd_step, L.gm_oracle_adam_step, L.gm_oracle_rmsprop_step,
                    L.gm_oracle_adagrad_step, L.gm_oracle_adadelta_step, L.gm_oracle_nadam_step):
             fn.restype = None
+        pp = ctypes.POINTER(c_float_p)
+        L.gm_oracle_lbfgs_dot.argtypes = [pp, pp, ctypes.POINTER(sz), i, i, i]
+        L.gm_oracle_lbfgs_dot.restype = f
+        L.gm_oracle_lbfgs_step.argtypes = [pp] * 6 + [c_float_p, c_float_p, ctypes.POINTER(sz),
+                                                      i, i, i, i, f, i, c_float_p]
+        L.gm_oracle_lbfgs_step.restype = i
         L.gm_oracle_f32_to_f16.argtypes = [f]
         L.gm_oracle_f32_to_f16.restype = ctypes.c_uint16
         L.gm_oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
@@ -103,6 +109,33 @@ class Oracle:
     def nadam(self, w, g, m, v, lr, beta1, beta2, eps, weight_decay, step, nthreads=1):
         self.lib.gm_oracle_nadam_step(_fp(w), _fp(g), _fp(m), _fp(v), w.size, lr, beta1, beta2, eps,
                                       weight_decay, step, nthreads)
+
+    # ---- L-BFGS ----
+    DOT_REFERENCE, DOT_TREE = 0, 1
+
+    def lbfgs_dot(self, a, b, mode, per_tensor=True):
+        """a, b: lists of float32 arrays."""
+        k = len(a)
+        P = (c_float_p * k)
+        sizes = (ctypes.c_size_t * k)(*[t.size for t in a])
+        return np.float32(self.lib.gm_oracle_lbfgs_dot(P(*[_fp(t) for t in a]), P(*[_fp(t) for t in b]),
+                                                       sizes, k, mode, 1 if per_tensor else 0))
+
+    def lbfgs_step(self, st, g, history_size, history_count, history_index, initial_step, mode):
+        """st: dict with lists of float32 arrays w, old_g, dir, s[h][i], y[h][i] and float32
+        arrays rho, alpha (history_size each); updated in place.  Returns (code, step_size)."""
+        k = len(g)
+        P = (c_float_p * k)
+        PH = (c_float_p * (k * history_size))
+        sizes = (ctypes.c_size_t * k)(*[t.size for t in g])
+        step = np.zeros(1, dtype=np.float32)
+        rc = self.lib.gm_oracle_lbfgs_step(
+            P(*[_fp(t) for t in st["w"]]), P(*[_fp(t) for t in g]), P(*[_fp(t) for t in st["old_g"]]),
+            P(*[_fp(t) for t in st["dir"]]),
+            PH(*[_fp(t) for h in st["s"] for t in h]), PH(*[_fp(t) for h in st["y"] for t in h]),
+            _fp(st["rho"]), _fp(st["alpha"]), sizes, k, history_size, history_count, history_index,
+            initial_step, mode, _fp(step))
+        return rc, float(step[0])
 
     # ---- casts ----
     def f32_to_f16(self, src, nthreads=1):
