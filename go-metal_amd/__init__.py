@@ -108,6 +108,21 @@ HOST_ABI = {
     "gmo_step_amp": (i, [u, up, up, i, ip]),
     "gmo_loss_scale": (f, [u]),
     "gmo_growth_tracker": (i, [u]),
+    "gmo_lbfgs_default_config": (None, [ip, fp, ip, fp, fp, fp]),
+    "gmo_lbfgs_new": (u, [i, f, i, f, f, f, ip, ip, i, u, u]),
+    "gmo_lbfgs_free": (None, [u]),
+    "gmo_lbfgs_set_weight_buffers": (i, [u, up, i]),
+    "gmo_lbfgs_step": (i, [u, up, i, f]),
+    "gmo_lbfgs_set_command_pool": (None, [u, u]),
+    "gmo_lbfgs_uses_pooling": (i, [u]),
+    "gmo_lbfgs_get_step": (ctypes.c_uint64, [u]),
+    "gmo_lbfgs_get_stats": (None, [u, ctypes.POINTER(ctypes.c_uint64), ip, ip, fp]),
+    "gmo_lbfgs_history": (None, [u, ip, ip, fp]),
+    "gmo_lbfgs_cleanup": (None, [u]),
+    "gmo_lbfgs_update_learning_rate": (i, [u, f]),
+    "gmo_lbfgs_set_log_progress": (None, [u, i]),
+    "gmo_lbfgs_buffer_size": (i, [u, i]),
+    "gmo_lbfgs_buffer": (u, [u, c_str, i, i]),
     "gmo_tensor_new": (u, [ip, i, i, i]),
     "gmo_tensor_retain": (u, [u]),
     "gmo_tensor_release": (None, [u]),
@@ -235,6 +250,80 @@ class Device:
         self._owned.clear()
         if self.handle:
             self.lib.destroy_metal_device(self.handle)
+            self.handle = 0
+
+
+class HostLBFGS:
+    """Python handle on the C++ LBFGSOptimizerState (mirror of optimizer/lbfgs.go)."""
+
+    def __init__(self, config, weight_shapes, memory_manager, device):
+        """config: (HistorySize, LineSearchTol, MaxLineSearch, C1, C2, InitialStep)."""
+        self.lib = load_library()
+        dims = [int(d) for shape in weight_shapes for d in shape]
+        ndims = [len(shape) for shape in weight_shapes]
+        hs, tol, mls, c1, c2, step = config
+        self.handle = self.lib.gmo_lbfgs_new(
+            int(hs), tol, int(mls), c1, c2, step, int_array(dims) if dims else None,
+            int_array(ndims) if ndims else None, len(weight_shapes), int(memory_manager or 0), int(device or 0))
+        self.error = None if self.handle else self.lib.gmo_last_error().decode()
+        if self.handle:
+            self.lib.gmo_lbfgs_set_log_progress(self.handle, 0)
+
+    @staticmethod
+    def default_config():
+        lib = load_library()
+        hs, mls = ctypes.c_int(), ctypes.c_int()
+        tol, c1, c2, step = f(), f(), f(), f()
+        lib.gmo_lbfgs_default_config(ctypes.byref(hs), ctypes.byref(tol), ctypes.byref(mls), ctypes.byref(c1),
+                                     ctypes.byref(c2), ctypes.byref(step))
+        return hs.value, tol.value, mls.value, c1.value, c2.value, step.value
+
+    def _err(self, rc):
+        return None if rc == 0 else self.lib.gmo_last_error().decode()
+
+    def SetWeightBuffers(self, buffers):
+        return self._err(self.lib.gmo_lbfgs_set_weight_buffers(self.handle, handle_array(buffers), len(buffers)))
+
+    def Step(self, gradient_buffers, current_loss):
+        return self._err(self.lib.gmo_lbfgs_step(self.handle, handle_array(gradient_buffers),
+                                                 len(gradient_buffers), current_loss))
+
+    def SetCommandPool(self, pool):
+        self.lib.gmo_lbfgs_set_command_pool(self.handle, int(pool or 0))
+
+    def uses_pooling(self):
+        return bool(self.lib.gmo_lbfgs_uses_pooling(self.handle))
+
+    def GetStep(self):
+        return self.lib.gmo_lbfgs_get_step(self.handle)
+
+    def GetStats(self):
+        step, hs, used, loss = ctypes.c_uint64(), ctypes.c_int(), ctypes.c_int(), f()
+        self.lib.gmo_lbfgs_get_stats(self.handle, ctypes.byref(step), ctypes.byref(hs), ctypes.byref(used),
+                                     ctypes.byref(loss))
+        return {"step": step.value, "history_size": hs.value, "history_used": used.value,
+                "prev_loss": loss.value}
+
+    def history(self):
+        count, index, step = ctypes.c_int(), ctypes.c_int(), f()
+        self.lib.gmo_lbfgs_history(self.handle, ctypes.byref(count), ctypes.byref(index), ctypes.byref(step))
+        return count.value, index.value, step.value
+
+    def UpdateLearningRate(self, lr):
+        return self._err(self.lib.gmo_lbfgs_update_learning_rate(self.handle, lr))
+
+    def Cleanup(self):
+        self.lib.gmo_lbfgs_cleanup(self.handle)
+
+    def buffer(self, which, history=0, index=0):
+        return self.lib.gmo_lbfgs_buffer(self.handle, which.encode(), history, index)
+
+    def buffer_size(self, index):
+        return self.lib.gmo_lbfgs_buffer_size(self.handle, index)
+
+    def free(self):
+        if self.handle:
+            self.lib.gmo_lbfgs_free(self.handle)
             self.handle = 0
 
 

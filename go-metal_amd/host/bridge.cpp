@@ -312,6 +312,54 @@ Error ExecuteNadamStepMPSGraph(Pointer device, const std::vector<Pointer> &weigh
     return "";
 }
 
+std::pair<float, Error> ExecuteLBFGSStepMPSGraph(
+    Pointer device, const std::vector<Pointer> &weightBuffers, const std::vector<Pointer> &gradientBuffers,
+    const std::vector<Pointer> &oldGradientBuffers, const std::vector<Pointer> &searchDirBuffers,
+    const std::vector<std::vector<Pointer>> &sVectors, const std::vector<std::vector<Pointer>> &yVectors,
+    const std::vector<Pointer> &rhoBuffers, Pointer alphaBuffer, int numWeights,
+    const std::vector<int> &bufferSizes, int historySize, int historyCount, int historyIndex,
+    float initialStep, float c1, float c2, int maxLineSearch, float currentLoss, float prevLoss,
+    Pointer commandPool, bool usePooling)
+{
+    // bridge.go:1963-1970
+    const size_t n = numWeights > 0 ? (size_t)numWeights : 0;
+    if (weightBuffers.size() != n || gradientBuffers.size() != n || oldGradientBuffers.size() != n ||
+        searchDirBuffers.size() != n || bufferSizes.size() != n || numWeights < 0)
+        return {0.0f, Errorf("buffer arrays must have length %d", numWeights)};
+    if (n == 0) return {0.0f, Errorf("%s", kEmptyList)};
+    // Go would panic indexing a short history slice; here it is an error.
+    if (historySize <= 0 || sVectors.size() != (size_t)historySize || yVectors.size() != (size_t)historySize ||
+        rhoBuffers.size() != (size_t)historySize)
+        return {0.0f, Errorf("history arrays must have length %d", historySize)};
+    auto w = handles(weightBuffers, n), g = handles(gradientBuffers, n), o = handles(oldGradientBuffers, n),
+         d = handles(searchDirBuffers, n), rho = handles(rhoBuffers, (size_t)historySize);
+    // flattened [hist0_weight0, hist0_weight1, ..., hist1_weight0, ...]  (bridge.go:1988-1999)
+    std::vector<uintptr_t> sFlat((size_t)historySize * n), yFlat((size_t)historySize * n);
+    for (int h = 0; h < historySize; h++) {
+        if (sVectors[h].size() != n || yVectors[h].size() != n)
+            return {0.0f, Errorf("history arrays must have %d buffers per entry", numWeights)};
+        for (size_t i = 0; i < n; i++) {
+            sFlat[(size_t)h * n + i] = reinterpret_cast<uintptr_t>(sVectors[h][i]);
+            yFlat[(size_t)h * n + i] = reinterpret_cast<uintptr_t>(yVectors[h][i]);
+        }
+    }
+    std::vector<int> sizes(bufferSizes);
+    float stepSize = 0.0f;
+    int result;
+    if (usePooling && commandPool != nullptr)
+        result = execute_lbfgs_step_mpsgraph_pooled(
+            H(device), w.data(), g.data(), o.data(), d.data(), sFlat.data(), yFlat.data(), rho.data(),
+            H(alphaBuffer), numWeights, sizes.data(), historySize, historyCount, historyIndex, initialStep, c1,
+            c2, maxLineSearch, currentLoss, prevLoss, H(commandPool), &stepSize);
+    else
+        result = execute_lbfgs_step_mpsgraph(
+            H(device), w.data(), g.data(), o.data(), d.data(), sFlat.data(), yFlat.data(), rho.data(),
+            H(alphaBuffer), numWeights, sizes.data(), historySize, historyCount, historyIndex, initialStep, c1,
+            c2, maxLineSearch, currentLoss, prevLoss, &stepSize);
+    if (result != 0) return {0.0f, Errorf("L-BFGS MPSGraph step failed with error code: %d", result)};
+    return {stepSize, ""};
+}
+
 Error ExecuteAdamAMPStep(Pointer device, const std::vector<Pointer> &weightBuffers,
                          const std::vector<Pointer> &gradient16Buffers,
                          const std::vector<Pointer> &momentumBuffers,

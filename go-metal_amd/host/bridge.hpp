@@ -89,6 +89,16 @@ Error ExecuteNadamStepMPSGraph(Pointer device, const std::vector<Pointer> &weigh
                                float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
                                int stepCount);
 
+// bridge.go:1939.  sVectors / yVectors are [historySize][numWeights]; returns the step size.
+std::pair<float, Error> ExecuteLBFGSStepMPSGraph(
+    Pointer device, const std::vector<Pointer> &weightBuffers, const std::vector<Pointer> &gradientBuffers,
+    const std::vector<Pointer> &oldGradientBuffers, const std::vector<Pointer> &searchDirBuffers,
+    const std::vector<std::vector<Pointer>> &sVectors, const std::vector<std::vector<Pointer>> &yVectors,
+    const std::vector<Pointer> &rhoBuffers, Pointer alphaBuffer, int numWeights,
+    const std::vector<int> &bufferSizes, int historySize, int historyCount, int historyIndex,
+    float initialStep, float c1, float c2, int maxLineSearch, float currentLoss, float prevLoss,
+    Pointer commandPool, bool usePooling);
+
 // Addition (no Go counterpart): the mixed-precision Adam step.  weight16Buffers may be
 // empty.  On success *skipped tells whether the step was dropped for an inf / NaN gradient.
 Error ExecuteAdamAMPStep(Pointer device, const std::vector<Pointer> &weightBuffers,

@@ -1,4 +1,5 @@
 // Flat C view of the host-side mirror (include/gometal_optimizer.h).
+#include "lbfgs.hpp"
 #include "optimizer.hpp"
 #include "scheduler.hpp"
 #include "tensor.hpp"
@@ -409,6 +410,113 @@ int gmo_growth_tracker(uintptr_t opt)
 {
     auto *a = adam_of(opt);
     return a ? a->GrowthTracker : -1;
+}
+
+// ---- optimizer/lbfgs.go ----
+static LBFGSOptimizerState *L(uintptr_t h) { return reinterpret_cast<LBFGSOptimizerState *>(h); }
+
+void gmo_lbfgs_default_config(int *history_size, float *line_search_tol, int *max_line_search, float *c1,
+                              float *c2, float *initial_step)
+{
+    const LBFGSConfig d = DefaultLBFGSConfig();
+    if (history_size) *history_size = d.HistorySize;
+    if (line_search_tol) *line_search_tol = d.LineSearchTol;
+    if (max_line_search) *max_line_search = d.MaxLineSearch;
+    if (c1) *c1 = d.C1;
+    if (c2) *c2 = d.C2;
+    if (initial_step) *initial_step = d.InitialStep;
+}
+
+uintptr_t gmo_lbfgs_new(int history_size, float line_search_tol, int max_line_search, float c1, float c2,
+                        float initial_step, const int *dims, const int *ndims, int num_weights,
+                        uintptr_t memory_manager, uintptr_t device)
+{
+    Shapes shapes;
+    const int *d = dims;
+    for (int k = 0; k < num_weights; k++) {
+        shapes.emplace_back(d, d + ndims[k]);
+        d += ndims[k];
+    }
+    auto [opt, err] = NewLBFGSOptimizer(LBFGSConfig{history_size, line_search_tol, max_line_search, c1, c2,
+                                                    initial_step},
+                                        shapes, MM(memory_manager), reinterpret_cast<Pointer>(device));
+    if (!err.empty()) {
+        fail(err);
+        return 0;
+    }
+    ok();
+    return reinterpret_cast<uintptr_t>(opt.release());
+}
+
+void gmo_lbfgs_free(uintptr_t lbfgs) { delete L(lbfgs); }
+
+int gmo_lbfgs_set_weight_buffers(uintptr_t lbfgs, const uintptr_t *buffers, int n)
+{
+    Error e = L(lbfgs)->SetWeightBuffers(pointers(buffers, n));
+    return e.empty() ? ok() : fail(e);
+}
+
+int gmo_lbfgs_step(uintptr_t lbfgs, const uintptr_t *gradient_buffers, int n, float current_loss)
+{
+    Error e = L(lbfgs)->Step(pointers(gradient_buffers, n), current_loss);
+    return e.empty() ? ok() : fail(e);
+}
+
+void gmo_lbfgs_set_command_pool(uintptr_t lbfgs, uintptr_t pool)
+{
+    L(lbfgs)->SetCommandPool(reinterpret_cast<Pointer>(pool));
+}
+
+int gmo_lbfgs_uses_pooling(uintptr_t lbfgs) { return L(lbfgs)->usePooling ? 1 : 0; }
+uint64_t gmo_lbfgs_get_step(uintptr_t lbfgs) { return L(lbfgs)->GetStep(); }
+
+void gmo_lbfgs_get_stats(uintptr_t lbfgs, uint64_t *step, int *history_size, int *history_used, float *prev_loss)
+{
+    auto stats = L(lbfgs)->GetStats();
+    if (step) *step = std::get<uint64_t>(stats.at("step"));
+    if (history_size) *history_size = (int)std::get<uint64_t>(stats.at("history_size"));
+    if (history_used) *history_used = (int)std::get<uint64_t>(stats.at("history_used"));
+    if (prev_loss) *prev_loss = std::get<float>(stats.at("prev_loss"));
+}
+
+void gmo_lbfgs_history(uintptr_t lbfgs, int *count, int *index, float *last_step_size)
+{
+    if (count) *count = L(lbfgs)->historyCount;
+    if (index) *index = L(lbfgs)->historyIndex;
+    if (last_step_size) *last_step_size = L(lbfgs)->lastStepSize;
+}
+
+void gmo_lbfgs_cleanup(uintptr_t lbfgs) { L(lbfgs)->Cleanup(); }
+
+int gmo_lbfgs_update_learning_rate(uintptr_t lbfgs, float lr)
+{
+    Error e = L(lbfgs)->UpdateLearningRate(lr);
+    return e.empty() ? ok() : fail(e);
+}
+
+void gmo_lbfgs_set_log_progress(uintptr_t lbfgs, int on) { L(lbfgs)->logProgress = on != 0; }
+
+int gmo_lbfgs_buffer_size(uintptr_t lbfgs, int index)
+{
+    auto *l = L(lbfgs);
+    return index >= 0 && (size_t)index < l->bufferSizes.size() ? l->bufferSizes[index] : -1;
+}
+
+uintptr_t gmo_lbfgs_buffer(uintptr_t lbfgs, const char *which, int history, int index)
+{
+    auto *l = L(lbfgs);
+    const std::string w = which ? which : "";
+    const bool h_ok = history >= 0 && history < l->config.HistorySize;
+    const bool i_ok = index >= 0 && (size_t)index < l->WeightBuffers.size();
+    Pointer p = nullptr;
+    if (w == "s" && h_ok && i_ok) p = l->sVectors[history][index];
+    else if (w == "y" && h_ok && i_ok) p = l->yVectors[history][index];
+    else if (w == "rho" && h_ok) p = l->rhoBuffers[history];
+    else if (w == "alpha") p = l->alphaBuffer;
+    else if (w == "old_gradient" && i_ok) p = l->oldGradients[index];
+    else if (w == "search_dir" && i_ok) p = l->searchDir[index];
+    else if (w == "weight" && i_ok) p = l->WeightBuffers[index];
+    return reinterpret_cast<uintptr_t>(p);
 }
 
 static memory::Tensor *T(uintptr_t h) { return reinterpret_cast<memory::Tensor *>(h); }

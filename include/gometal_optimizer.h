@@ -87,6 +87,29 @@ int   gmo_step_amp(uintptr_t adam, const uintptr_t *gradient16_buffers, const ui
 float gmo_loss_scale(uintptr_t adam);
 int   gmo_growth_tracker(uintptr_t adam);
 
+/* ---- optimizer/lbfgs.go: LBFGSOptimizerState (not an optimizer.Optimizer in the reference
+ * either: Step also takes the current loss).  Errors as above: -1 / 0 and gmo_last_error(). ---- */
+void      gmo_lbfgs_default_config(int *history_size, float *line_search_tol, int *max_line_search, float *c1,
+                                   float *c2, float *initial_step);            /* DefaultLBFGSConfig, lbfgs.go:55 */
+uintptr_t gmo_lbfgs_new(int history_size, float line_search_tol, int max_line_search, float c1, float c2,
+                        float initial_step, const int *dims, const int *ndims, int num_weights,
+                        uintptr_t memory_manager, uintptr_t device);           /* NewLBFGSOptimizer, lbfgs.go:67 */
+void      gmo_lbfgs_free(uintptr_t lbfgs);
+int       gmo_lbfgs_set_weight_buffers(uintptr_t lbfgs, const uintptr_t *buffers, int n);   /* lbfgs.go:235 */
+int       gmo_lbfgs_step(uintptr_t lbfgs, const uintptr_t *gradient_buffers, int n, float current_loss); /* :245 */
+void      gmo_lbfgs_set_command_pool(uintptr_t lbfgs, uintptr_t pool);         /* lbfgs.go:304 */
+int       gmo_lbfgs_uses_pooling(uintptr_t lbfgs);
+uint64_t  gmo_lbfgs_get_step(uintptr_t lbfgs);                                 /* lbfgs.go:310 */
+void      gmo_lbfgs_get_stats(uintptr_t lbfgs, uint64_t *step, int *history_size, int *history_used,
+                              float *prev_loss);                               /* GetStats, lbfgs.go:315 */
+void      gmo_lbfgs_history(uintptr_t lbfgs, int *count, int *index, float *last_step_size);
+void      gmo_lbfgs_cleanup(uintptr_t lbfgs);                                  /* lbfgs.go:325 */
+int       gmo_lbfgs_update_learning_rate(uintptr_t lbfgs, float lr);           /* always an error, lbfgs.go:330 */
+void      gmo_lbfgs_set_log_progress(uintptr_t lbfgs, int on);
+int       gmo_lbfgs_buffer_size(uintptr_t lbfgs, int index);                   /* bytes; -1 if out of range */
+/* which: "s", "y" (history, index), "rho" (history), "alpha", "old_gradient", "search_dir", "weight" (index) */
+uintptr_t gmo_lbfgs_buffer(uintptr_t lbfgs, const char *which, int history, int index);
+
 /* ---- memory.Tensor (memory/tensor.go): reference-counted tensor over a pooled buffer.
  * dtype codes: Float32 = 0, Int32 = 1, Float16 = 2, Int8 = 3 (tensor.go:10-17). ---- */
 uintptr_t gmo_tensor_new(const int *shape, int ndims, int dtype, int device_type);   /* NewTensor, tensor.go:41 */

@@ -290,3 +290,21 @@ def test_lr_schedulers_follow_the_reference_formulas(vanilla_sgd):
     assert vanilla_sgd.field("LearningRate") == f32(0.01 * math.pow(0.95, 3.0))
     for h in (step, bad, expo, cos, plateau, const):
         lib.gmo_scheduler_free(h)
+
+
+# ---- optimizer/lbfgs.go without a GPU: lbfgs_test.go:11-32, 131-162 and the Go error strings ----
+def test_lbfgs_default_config_and_constructor_errors(mm):
+    cfg = pkg.HostLBFGS.default_config()
+    assert cfg == (10, f32(1e-4), 20, f32(1e-4), f32(0.9), 1.0)
+    assert pkg.HostLBFGS(cfg, [[10, 5]], 0, MOCK_DEVICE).error == "memory manager cannot be nil"
+    assert pkg.HostLBFGS(cfg, [[10, 5]], mm, 0).error == "device cannot be nil"
+    assert pkg.HostLBFGS(cfg, [], mm, MOCK_DEVICE).error == "no weight shapes provided"
+    assert pkg.HostLBFGS((0,) + cfg[1:], [[10, 5]], mm, MOCK_DEVICE).error == \
+        "history size must be positive, got 0"
+    # without a GPU behind the manager the first allocation fails and everything is released
+    opt = pkg.HostLBFGS(cfg, [[10, 5]], mm, MOCK_DEVICE)
+    if lib.create_metal_device() == 0:
+        assert opt.error == "failed to allocate s vector buffer for history 0, weight 0"
+    else:
+        opt.Cleanup()
+        opt.free()
