@@ -110,12 +110,132 @@ def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_
                       f"{dt:.1f} s, oracle/oracle.c with OpenMP on {threads} threads"}
 
 
+LBFGS_WORKLOADS = {
+    # name: (description, sizes(), history size)
+    "lbfgs-c3": ("L-BFGS, history 10 (all pairs valid), 25M params in 160 ragged tensors", ragged_sizes, 10),
+    "lbfgs-c5": ("L-BFGS, history 10 (all pairs valid), 1,012,301,824 params in 400 transformer-block tensors",
+                 transformer_block_sizes, 10),
+}
+
+
+def lbfgs_bytes_per_param(valid_pairs):
+    """Algorithmic HBM bytes per parameter of one L-BFGS step with a non-empty history: every pass reads
+    its operands once and writes its result once.  No valid pair: update (g, w -> p, w, old_g, s: 24) +
+    curvature (g, old_g, s -> y: 16).  c valid pairs: init (12) + c backward (16) + c forward (16, the last one 12) +
+    update (28) + curvature (16)."""
+    c = valid_pairs
+    return 40 if c == 0 else 12 + 16 * c + 16 * c - 4 + 28 + 16
+
+
+def bench_lbfgs(args, pkg, dev):
+    lib, D = dev.lib, dev.handle
+    desc, sizes_fn, m = LBFGS_WORKLOADS[args.workload]
+    sizes = sizes_fn()
+    n, params = len(sizes), sum(sizes)
+    fill = lambda h, k, seed, std: lib.gm_fill_normal_f32(D, h, k, seed, 0.0, std)
+
+    def tensor_list(seed, std):
+        hs = [dev.alloc(4 * k) for k in sizes]
+        for i, k in enumerate(sizes):
+            fill(hs[i], k, seed + i, std)
+        return hs
+
+    w, g = tensor_list(0x1000, 0.02), tensor_list(0x2000, 1e-2)
+    old_g, direction = tensor_list(0x3000, 1e-2), tensor_list(0x4000, 1e-2)
+    s = [tensor_list(0x10000 * (h + 1), 1e-2) for h in range(m)]
+    y = [tensor_list(0x10000 * (h + 1) + 0x8000, 1e-2) for h in range(m)]
+    rho_value = np.full(1, 1e-3, np.float32)
+    rho = [dev.from_numpy(rho_value) for _ in range(m)]
+    alpha = dev.alloc(4 * m, zero=True)
+    dev.synchronize()
+    arr = pkg.handle_array
+    cw, cg, co, cd = arr(w), arr(g), arr(old_g), arr(direction)
+    cs, cy, cr = arr([b for h in s for b in h]), arr([b for h in y for b in h]), arr(rho)
+    bs = pkg.int_array([4 * k for k in sizes])
+    step_size = ctypes.c_float()
+    state = {"index": 0}
+
+    def launch(count, valid=True):
+        # a step with index i ends by clearing rho[i - 1] (its y is g - g); put the value back before the
+        # next step so that every pair stays valid
+        idx = state["index"]
+        if count and valid:
+            dev.upload(rho[(idx - 2) % m], rho_value)
+        rc = lib.execute_lbfgs_step_mpsgraph(D, cw, cg, co, cd, cs, cy, cr, alpha, n, bs, m, count, idx, 0.01,
+                                             1e-4, 0.9, 20, 1.0, 1.0, ctypes.byref(step_size))
+        if rc != 0:
+            raise RuntimeError(f"L-BFGS step failed rc={rc}: {lib.gm_last_error().decode()}")
+        state["index"] = (idx + 1) % m
+
+    full_wall, full_event = time_steps(dev, lambda: launch(m), args.steps, args.warmup)
+    live = sum(1 for h in rho if dev.to_numpy(h, 1)[0] != 0.0)
+    if live < m - 1:
+        raise RuntimeError(f"only {live} of {m} history pairs stayed valid during the timed steps")
+    # the history the reference's own optimizer produces: every rho is 0, a step is update + curvature
+    for h in rho:
+        dev.upload(h, np.zeros(1, np.float32))
+    plain_wall, plain_event = time_steps(dev, lambda: launch(m, valid=False), args.steps, args.warmup)
+    bpp = lbfgs_bytes_per_param(m)
+    achieved = params * bpp / (full_event * 1e-3) / 1e9
+    plain = params * lbfgs_bytes_per_param(0) / (plain_event * 1e-3) / 1e9
+    result = {
+        "metric": f"params updated/sec (L-BFGS step, {m} history pairs) + achieved HBM GB/s",
+        "value": params / (full_wall * 1e-3), "unit": "params/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": full_wall, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 (dot products accumulated in f64)", "data": "synthetic",
+        "config": {"workload": desc, "tensors": n, "params": params, "rule": "lbfgs", "history_size": m},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "lbfgs_stream_kernel (all passes)",
+                     "bytes_per_param": bpp, "kernel_ms": full_event,
+                     "note": "time covers every pass of the step, the tree reductions between them and the "
+                             "read-back of the pair flags"},
+        "all_pairs_invalid_step": {"ms_per_step": plain_wall, "bytes_per_param": lbfgs_bytes_per_param(0),
+                               "achieved": plain, "frac": plain / HBM_PEAK_GBS},
+    }
+    if args.no_cpu_baseline:
+        result["cpu_baseline"] = None
+    else:
+        result["cpu_baseline"] = lbfgs_cpu_baseline(sizes, m)
+    dev.close()
+    print(json.dumps(result))
+
+
+def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
+    """The reference's algorithm as it runs it: one CPU thread, running fp32 sums
+    (oracle/oracle_lbfgs.c in reference order), on the leading tensors of the workload."""
+    from oracle_lib import oracle
+    o = oracle()
+    chosen, total = [], 0
+    for k in sizes:
+        if chosen and total + k > budget_params:
+            break
+        chosen.append(k)
+        total += k
+    rng = np.random.default_rng(1)
+    r = lambda std: [rng.standard_normal(k, dtype=np.float32) * np.float32(std) for k in chosen]
+    st = {"w": r(0.02), "old_g": r(1e-2), "dir": r(1e-2), "s": [r(1e-2) for _ in range(m)],
+          "y": [r(1e-2) for _ in range(m)], "rho": np.full(m, 1e-3, np.float32), "alpha": np.zeros(m, np.float32)}
+    g = r(1e-2)
+    steps, index, dt = 0, 0, 0.0
+    while dt < target_seconds and steps < 2000:
+        st["rho"][:] = 1e-3
+        t0 = time.perf_counter()
+        o.lbfgs_step(st, g, m, m, index, 0.01, 0)
+        dt += time.perf_counter() - t0
+        index = (index + 1) % m
+        steps += 1
+    return {"value": total * steps / dt, "unit": "params/s", "cores": 1, "kind": "port",
+            "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} steps in {dt:.1f} s, "
+                      "oracle/oracle_lbfgs.c in the reference's summation order on one thread (the reference "
+                      "runs this step as a single-threaded CPU loop)"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
     # launch-shape overrides (gm_set_tuning) for comparing lane widths and chunk sizes; 0 / -1 = default
@@ -133,6 +253,9 @@ def main():
     lib, D = dev.lib, dev.handle
     if lib.gm_set_tuning(args.chunk, args.nontemporal, args.vec) != 0:
         sys.exit("invalid --chunk / --vec combination (a chunk is a power-of-two multiple of 256 * vec elements)")
+
+    if args.workload in LBFGS_WORKLOADS:
+        return bench_lbfgs(args, pkg, dev)
 
     desc, sizes_fn, rule, hyper, grad_std = WORKLOADS[args.workload]
     sizes = sizes_fn()
