@@ -210,7 +210,7 @@ __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
     // Order of a lane's memory operations: element by element, all loads of the element, then
     // its stores.  The compiler cannot prove that the streams do not overlap, so a store orders
     // the loads around it; a store placed between two loads of one element leaves a single load
-    // in flight per lane (the init pass ran at 53 % of peak that way, 71 % with loads first).
+    // in flight per lane (the init pass ran at 53 % of peak that way, 75 % with loads first).
     // Hoisting the loads of all four elements above the first store is slower for the passes
     // that feed a dot product (68 % against 86 % of peak): reads and writes then reach the
     // memory controllers in bursts instead of finely interleaved.

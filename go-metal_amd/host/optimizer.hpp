@@ -1,7 +1,7 @@
 // Host-side mirror of the Go package `optimizer` (optimizer/*.go): the state objects that
 // own hyper-parameters, step counters and device-resident state buffers, and drive the C ABI.
 // Type names, method names, argument meaning, validation order and error strings follow the
-// Go sources; an empty Error is Go's nil.  L-BFGS is not part of this path.
+// Go sources; an empty Error is Go's nil.  L-BFGS lives in lbfgs.hpp.
 #pragma once
 
 #include "bridge.hpp"
