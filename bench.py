@@ -34,7 +34,9 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
-MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10}
+MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10,
+                        # bytes per step, summed over the passes of a 10-pair step (profiles/lbfgs_c5_1b_hbm_traffic.md)
+                        ("lbfgs-c5", 10): 368.72 * 1012301824}
 
 from workloads import amp_125m_sizes, cnn_sizes, ragged_sizes, transformer_block_sizes  # noqa: E402
 
@@ -121,15 +123,19 @@ LBFGS_WORKLOADS = {
 def lbfgs_bytes_per_param(valid_pairs):
     """Algorithmic HBM bytes per parameter of one L-BFGS step with a non-empty history: every pass reads
     its operands once and writes its result once.  No valid pair: update (g, w -> p, w, old_g, s: 24) +
-    curvature (g, old_g, s -> y: 16).  c valid pairs: init (12) + c backward (16) + c forward (16, the last one 12) +
-    update (28) + curvature (16)."""
+    curvature (g, old_g, s -> y: 16).  c valid pairs: init (12) + c backward (16; the last one 12, its dot
+    operand y_0 being the buffer its axpy reads) + c forward (16; the last one 12, no dot) + update (28) +
+    curvature (16)."""
     c = valid_pairs
-    return 40 if c == 0 else 12 + 16 * c + 16 * c - 4 + 28 + 16
+    return 40 if c == 0 else 12 + (16 * c - 4) + (16 * c - 4) + 28 + 16
 
 
 def bench_lbfgs(args, pkg, dev):
     lib, D = dev.lib, dev.handle
     desc, sizes_fn, m = LBFGS_WORKLOADS[args.workload]
+    if args.history > 0:
+        desc = desc.replace(f"history {m}", f"history {args.history}")
+        m = args.history
     sizes = sizes_fn()
     n, params = len(sizes), sum(sizes)
     fill = lambda h, k, seed, std: lib.gm_fill_normal_f32(D, h, k, seed, 0.0, std)
@@ -138,6 +144,7 @@ def bench_lbfgs(args, pkg, dev):
         hs = [dev.alloc(4 * k) for k in sizes]
         for i, k in enumerate(sizes):
             fill(hs[i], k, seed + i, std)
+        print(f"filled a list of {len(sizes)} tensors", file=sys.stderr, flush=True)
         return hs
 
     w, g = tensor_list(0x1000, 0.02), tensor_list(0x2000, 1e-2)
@@ -185,7 +192,8 @@ def bench_lbfgs(args, pkg, dev):
         "vs_baseline": None, "dtype": "f32 (dot products accumulated in f64)", "data": "synthetic",
         "config": {"workload": desc, "tensors": n, "params": params, "rule": "lbfgs", "history_size": m},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "lbfgs_stream_kernel (all passes)",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_HBM_TRAFFIC.get((args.workload, m)),
+                     "kernel": "lbfgs_stream_kernel (all passes)",
                      "bytes_per_param": bpp, "kernel_ms": full_event,
                      "note": "time covers every pass of the step, the tree reductions between them and the "
                              "read-back of the pair flags"},
@@ -238,6 +246,7 @@ def main():
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
+    ap.add_argument("--history", type=int, default=0, help="L-BFGS workloads: history size (default 10)")
     # launch-shape overrides (gm_set_tuning) for comparing lane widths and chunk sizes; 0 / -1 = default
     ap.add_argument("--chunk", type=int, default=0, help="elements per chunk")
     ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4")
