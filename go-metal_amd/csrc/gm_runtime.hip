@@ -105,7 +105,9 @@ typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(256)
 convert_f32_to_f16_kernel(const float *__restrict__ src, __half *__restrict__ dst, size_t n)
 {
-    const size_t n4 = n / 4;
+    // 4-element groups only when both views are aligned for them (handles may be offset addresses)
+    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 8 == 0;
+    const size_t n4 = aligned ? n / 4 : 0;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
         floatx4 x = reinterpret_cast<const floatx4 *>(src)[i];
@@ -116,15 +118,15 @@ convert_f32_to_f16_kernel(const float *__restrict__ src, __half *__restrict__ ds
         packed.y = *reinterpret_cast<unsigned int *>(&hi);
         reinterpret_cast<uint2 *>(dst)[i] = packed;
     }
-    if (blockIdx.x == 0) {
-        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += blockDim.x) dst[i] = __float2half_rn(src[i]);
-    }
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        dst[i] = __float2half_rn(src[i]);
 }
 
 __global__ void __launch_bounds__(256)
 convert_f16_to_f32_kernel(const __half *__restrict__ src, float *__restrict__ dst, size_t n)
 {
-    const size_t n4 = n / 4;
+    const bool aligned = reinterpret_cast<uintptr_t>(src) % 8 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+    const size_t n4 = aligned ? n / 4 : 0;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
         uint2 packed = reinterpret_cast<const uint2 *>(src)[i];
@@ -137,9 +139,8 @@ convert_f16_to_f32_kernel(const __half *__restrict__ src, float *__restrict__ ds
         y.w = __high2float(hi);
         reinterpret_cast<floatx4 *>(dst)[i] = y;
     }
-    if (blockIdx.x == 0) {
-        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += blockDim.x) dst[i] = __half2float(src[i]);
-    }
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        dst[i] = __half2float(src[i]);
 }
 
 // Zero fill: 16-byte stores, byte tail.  (A kernel rather than hipMemsetAsync, so
@@ -147,13 +148,17 @@ convert_f16_to_f32_kernel(const __half *__restrict__ src, float *__restrict__ ds
 __global__ void __launch_bounds__(256)
 zero_kernel(unsigned char *__restrict__ dst, size_t bytes)
 {
-    const size_t n16 = bytes / 16;
+    // bytes up to the first 16-byte boundary, 16-byte stores, byte tail
+    size_t head = (16 - reinterpret_cast<uintptr_t>(dst) % 16) % 16;
+    if (head > bytes) head = bytes;
+    const size_t n16 = (bytes - head) / 16;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uintx4 z = {0u, 0u, 0u, 0u};
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
-        reinterpret_cast<uintx4 *>(dst)[i] = z;
+    for (size_t i = tid; i < n16; i += stride) reinterpret_cast<uintx4 *>(dst + head)[i] = z;
     if (blockIdx.x == 0) {
-        for (size_t i = n16 * 16 + threadIdx.x; i < bytes; i += blockDim.x) dst[i] = 0;
+        for (size_t i = threadIdx.x; i < head; i += blockDim.x) dst[i] = 0;
+        for (size_t i = head + n16 * 16 + threadIdx.x; i < bytes; i += blockDim.x) dst[i] = 0;
     }
 }
 
@@ -318,6 +323,11 @@ int zero_metal_buffer_mpsgraph(uintptr_t device, uintptr_t buffer, int size)
 int copy_data_to_metal_buffer(uintptr_t buffer, void *data, int size)
 {
     if (buffer == 0 || data == nullptr || size <= 0) return -1;
+    const size_t len = registry_length(buffer);
+    if (len != 0 && (size_t)size > len) {
+        set_error("copy of %d bytes exceeds the %zu-byte buffer", size, len);
+        return -3;
+    }
     Context *ctx = default_context();
     if (!ctx || !make_current(ctx)) return -4;
     // Pageable source: the call returns once the host range has been consumed,
@@ -345,6 +355,11 @@ int copy_int32_array_to_metal_buffer(uintptr_t buffer, int *data, int num_elemen
 
 static int copy_from_buffer(uintptr_t buffer, void *data, size_t bytes)
 {
+    const size_t len = registry_length(buffer);
+    if (len != 0 && bytes > len) {
+        set_error("read of %zu bytes exceeds the %zu-byte buffer", bytes, len);
+        return -3;
+    }
     Context *ctx = default_context();
     if (!ctx || !make_current(ctx)) return -4;
     if (!hip_ok(hipMemcpyAsync(data, reinterpret_cast<void *>(buffer), bytes, hipMemcpyDeviceToHost,
@@ -382,6 +397,13 @@ int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, 
     Context *ctx = resolve_device(device);
     if (!ctx || !make_current(ctx)) return -4;
     if (total == 0) return 0;
+    const size_t src_len = registry_length(src_buffer), dst_len = registry_length(dst_buffer);
+    if ((src_len != 0 && total * (to_half ? 4 : 2) > src_len) ||
+        (dst_len != 0 && total * (to_half ? 2 : 4) > dst_len)) {
+        set_error("conversion of %zu elements exceeds a buffer (src %zu bytes, dst %zu bytes)", total, src_len,
+                  dst_len);
+        return -5;
+    }
     const unsigned int grid = grid_for((total + 3) / 4, 256, 1u << 20);
     if (to_half)
         convert_f32_to_f16_kernel<<<grid, 256, 0, ctx->stream>>>(
@@ -489,8 +511,9 @@ int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, 
     if (!ctx) return -3;
     if (!make_current(ctx)) return -10;
     const size_t src_len = registry_length(src_buffer), dst_len = registry_length(dst_buffer);
-    if ((src_len != 0 && bytes > src_len) || (dst_len != 0 && bytes > dst_len) || bytes % 16 != 0) {
-        set_error("copy probe of %zu bytes does not fit (src %zu, dst %zu) or is not a multiple of 16",
+    if ((src_len != 0 && bytes > src_len) || (dst_len != 0 && bytes > dst_len) || bytes % 16 != 0 ||
+        src_buffer % 16 != 0 || dst_buffer % 16 != 0) {
+        set_error("copy probe of %zu bytes does not fit (src %zu, dst %zu) or is not 16-byte aligned and sized",
                   bytes, src_len, dst_len);
         return -5;
     }

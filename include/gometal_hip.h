@@ -65,19 +65,21 @@ void deallocate_metal_buffer(uintptr_t buffer);
 int zero_metal_buffer(uintptr_t device, uintptr_t buffer, int size);
 /* bridge_memory.m:58-160; same effect as zero_metal_buffer here. */
 int zero_metal_buffer_mpsgraph(uintptr_t device, uintptr_t buffer, int size);
-/* bridge_memory.m:191-218.  -1: nil buffer / NULL data / size <= 0; -4: HIP error. */
+/* bridge_memory.m:191-218.  -1: nil buffer / NULL data / size <= 0; -3: the range exceeds
+ * the allocation (buffers of this library only; the reference does not check); -4: HIP error. */
 int copy_data_to_metal_buffer(uintptr_t buffer, void *data, int size);
 /* bridge_memory.m:221-258.  -1: nil / NULL / n <= 0. */
 int copy_float32_array_to_metal_buffer(uintptr_t buffer, float *data, int num_elements);
 int copy_int32_array_to_metal_buffer(uintptr_t buffer, int *data, int num_elements);
-/* bridge_memory.m:261-320.  Synchronises the stream first.  -1 / -4 as above. */
+/* bridge_memory.m:261-320.  Synchronises the stream first.  -1 / -3 / -4 as above. */
 int copy_metal_buffer_to_float32_array(uintptr_t buffer, float *data, int num_elements);
 int copy_metal_buffer_to_int32_array(uintptr_t buffer, int *data, int num_elements);
 /* bridge_memory.m:323-423.  Element count = product of shape[0..num_dims).
  * Type codes from memory/tensor.go:12-17: Float32 = 0, Float16 = 2.
  * fp32->fp16 rounds to nearest even and overflows to +-inf; fp16->fp32 is
  * exact.  -1: nil buffers / NULL shape / num_dims <= 0; -2: nil device;
- * -3: any pair other than 0->2 or 2->0; -4: HIP error. */
+ * -3: any pair other than 0->2 or 2->0; -4: HIP error; -5: the element count exceeds
+ * one of the allocations (buffers of this library only). */
 int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, int num_dims,
                         int src_type, int dst_type, uintptr_t device);
 /* bridge_memory.m:504-592.  -1: nil handle; -2: size <= 0 or negative offset;

@@ -145,3 +145,53 @@ def test_fill_normal_is_reproducible_and_sane(dev):
     assert abs(xa.mean() - 0.5) < 0.02 and abs(xa.std() - 2.0) < 0.02 and np.all(np.isfinite(xa))
     dev.free(a)
     dev.free(b)
+
+
+def test_offset_views_take_the_unaligned_paths(dev):
+    """A handle is a device address, so a caller may pass base + offset: zeroing and the casts
+    must not assume 16-byte alignment, and must leave the bytes around the view alone."""
+    o = oracle()
+    n = 1000
+    x = (np.random.default_rng(5).standard_normal(n + 8) * 3).astype(np.float32)
+    src = dev.from_numpy(x)
+    dst16 = dev.from_numpy(np.full(n + 16, 0x1234, np.uint16))
+    shape = (ctypes.c_int * 1)(n - 3)
+    # fp32 view starting 4 bytes in, fp16 view starting 2 bytes in
+    assert dev.lib.convert_tensor_type(src + 4, dst16 + 2, shape, 1, 0, 2, dev.handle) == 0
+    got = dev.to_numpy(dst16, n + 16, np.uint16)
+    assert np.array_equal(got[1:n - 2], o.f32_to_f16(x[1:n - 2]))
+    assert got[0] == 0x1234 and np.all(got[n - 2:] == 0x1234)
+    # and back, into an fp32 view that is 4 bytes off
+    back = dev.from_numpy(np.full(n + 8, -7.0, np.float32))
+    assert dev.lib.convert_tensor_type(dst16 + 2, back + 4, shape, 1, 2, 0, dev.handle) == 0
+    got32 = dev.to_numpy(back, n + 8)
+    assert np.array_equal(got32[1:n - 2].view(np.uint32), o.f16_to_f32(got[1:n - 2]).view(np.uint32))
+    assert got32[0] == -7.0 and np.all(got32[n - 2:] == -7.0)
+    # zero 37 bytes starting 5 bytes in
+    raw = dev.from_numpy(np.full(64, 0xAB, np.uint8))
+    assert dev.lib.zero_metal_buffer(dev.handle, raw + 5, 37) == 0
+    b = dev.to_numpy(raw, 64, np.uint8)
+    assert np.all(b[:5] == 0xAB) and np.all(b[5:42] == 0) and np.all(b[42:] == 0xAB)
+    for h in (src, dst16, back, raw):
+        dev.free(h)
+
+
+def test_ranges_beyond_an_allocation_are_refused(dev):
+    """The reference trusts its callers here; an overrun on a GPU is a fault, so buffers of this
+    library are checked against their recorded length."""
+    buf = dev.alloc(64)
+    small = dev.alloc(16)
+    host = np.zeros(64, np.float32)
+    assert dev.lib.copy_float32_array_to_metal_buffer(buf, host.ctypes.data_as(vp), 17) == -3
+    assert dev.lib.copy_data_to_metal_buffer(buf, host.ctypes.data_as(vp), 65) == -3
+    assert dev.lib.copy_metal_buffer_to_float32_array(buf, host.ctypes.data_as(vp), 17) == -3
+    assert b"exceeds" in dev.lib.gm_last_error()
+    assert dev.lib.copy_float32_array_to_metal_buffer(buf, host.ctypes.data_as(vp), 16) == 0
+    shape = (ctypes.c_int * 1)(16)
+    assert dev.lib.convert_tensor_type(buf, small, shape, 1, 0, 2, dev.handle) == -5     # 32 bytes into 16
+    assert dev.lib.convert_tensor_type(small, buf, shape, 1, 2, 0, dev.handle) == -5     # 32 bytes out of 16
+    shape8 = (ctypes.c_int * 1)(8)
+    assert dev.lib.convert_tensor_type(buf, small, shape8, 1, 0, 2, dev.handle) == 0
+    assert dev.lib.zero_metal_buffer(dev.handle, buf, 65) == -5
+    dev.free(buf)
+    dev.free(small)
