@@ -191,23 +191,30 @@ void gmo_optimizer_free(uintptr_t opt) { delete H(opt); }
 
 int gmo_set_weight_buffers(uintptr_t opt, const uintptr_t *weight_buffers, int n)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     Error e = H(opt)->opt->SetWeightBuffers(pointers(weight_buffers, n));
     return e.empty() ? ok() : fail(e);
 }
 
 int gmo_step(uintptr_t opt, const uintptr_t *gradient_buffers, int n)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     Error e = H(opt)->opt->Step(pointers(gradient_buffers, n));
     return e.empty() ? ok() : fail(e);
 }
 
-uint64_t gmo_get_step_count(uintptr_t opt) { return H(opt)->opt->GetStepCount(); }
-void gmo_update_learning_rate(uintptr_t opt, float lr) { H(opt)->opt->UpdateLearningRate(lr); }
-void gmo_set_command_pool(uintptr_t opt, uintptr_t pool) { H(opt)->opt->SetCommandPool(reinterpret_cast<Pointer>(pool)); }
-void gmo_cleanup(uintptr_t opt) { H(opt)->opt->Cleanup(); }
+uint64_t gmo_get_step_count(uintptr_t opt) {
+    if (!opt) { fail(Errorf("object handle is nil")); return 0; } return H(opt)->opt->GetStepCount(); }
+void gmo_update_learning_rate(uintptr_t opt, float lr) {
+    if (!opt) return; H(opt)->opt->UpdateLearningRate(lr); }
+void gmo_set_command_pool(uintptr_t opt, uintptr_t pool) {
+    if (!opt) return; H(opt)->opt->SetCommandPool(reinterpret_cast<Pointer>(pool)); }
+void gmo_cleanup(uintptr_t opt) {
+    if (!opt) return; H(opt)->opt->Cleanup(); }
 
 char *gmo_get_state_json(uintptr_t opt)
 {
+    if (!opt) { fail(Errorf("object handle is nil")); return nullptr; }
     auto [state, err] = H(opt)->opt->GetState();
     if (!err.empty() || !state) {
         fail(err);
@@ -222,6 +229,7 @@ char *gmo_get_state_json(uintptr_t opt)
 
 int gmo_load_state_json(uintptr_t opt, const char *json)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     auto [state, perr] = OptimizerState::FromJSON(json ? json : "");
     if (!perr.empty()) return fail(perr);
     Error e = H(opt)->opt->LoadState(&state);
@@ -230,6 +238,7 @@ int gmo_load_state_json(uintptr_t opt, const char *json)
 
 char *gmo_get_checkpoint_json(uintptr_t opt)
 {
+    if (!opt) { fail(Errorf("object handle is nil")); return nullptr; }
     auto [state, err] = H(opt)->opt->GetState();
     if (!err.empty() || !state) {
         fail(err);
@@ -244,6 +253,7 @@ char *gmo_get_checkpoint_json(uintptr_t opt)
 
 int gmo_load_checkpoint_json(uintptr_t opt, const char *json)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     auto [state, perr] = OptimizerState::FromCheckpointJSON(json ? json : "");
     if (!perr.empty()) return fail(perr);
     Error e = H(opt)->opt->LoadState(&state);
@@ -252,6 +262,7 @@ int gmo_load_checkpoint_json(uintptr_t opt, const char *json)
 
 float gmo_get_field(uintptr_t opt, const char *name)
 {
+    if (!opt) return std::nanf("");
     Handle *h = H(opt);
     const std::string n = name ? name : "";
     auto b = [](bool v) { return v ? 1.0f : 0.0f; };
@@ -312,6 +323,7 @@ float gmo_get_field(uintptr_t opt, const char *name)
 
 uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index)
 {
+    if (!opt) { fail(Errorf("object handle is nil")); return 0; }
     Handle *h = H(opt);
     const std::string t = state_type ? state_type : "";
     const std::vector<Pointer> *v = nullptr;
@@ -354,6 +366,7 @@ uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index)
 
 int gmo_uses_pooling(uintptr_t opt)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     Handle *h = H(opt);
     switch (h->kind) {
     case GMO_SGD: return static_cast<SGDOptimizerState *>(h->opt.get())->usePooling;
@@ -368,6 +381,7 @@ int gmo_uses_pooling(uintptr_t opt)
 
 void gmo_set_log_progress(uintptr_t opt, int on)
 {
+    if (!opt) return;
     Handle *h = H(opt);
     if (h->kind == GMO_ADAGRAD) static_cast<AdaGradOptimizerState *>(h->opt.get())->logProgress = on != 0;
     if (h->kind == GMO_ADADELTA) static_cast<AdaDeltaOptimizerState *>(h->opt.get())->logProgress = on != 0;
@@ -383,6 +397,7 @@ static AdamOptimizerState *adam_of(uintptr_t opt)
 int gmo_enable_mixed_precision(uintptr_t opt, float initial_scale, float growth_factor, float backoff_factor,
                                int growth_interval)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     auto *a = adam_of(opt);
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
     Error e = a->EnableMixedPrecision(initial_scale, growth_factor, backoff_factor, growth_interval);
@@ -392,6 +407,7 @@ int gmo_enable_mixed_precision(uintptr_t opt, float initial_scale, float growth_
 int gmo_step_amp(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n,
                  int *skipped)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     auto *a = adam_of(opt);
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
     auto [sk, e] = a->StepAMP(pointers(gradient16_buffers, n), pointers(weight16_buffers, weight16_buffers ? n : 0));
@@ -402,12 +418,14 @@ int gmo_step_amp(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintp
 
 float gmo_loss_scale(uintptr_t opt)
 {
+    if (!opt) return std::nanf("");
     auto *a = adam_of(opt);
     return a ? a->LossScale : std::nanf("");
 }
 
 int gmo_growth_tracker(uintptr_t opt)
 {
+    if (!opt) return fail(Errorf("object handle is nil"));
     auto *a = adam_of(opt);
     return a ? a->GrowthTracker : -1;
 }
@@ -452,26 +470,32 @@ void gmo_lbfgs_free(uintptr_t lbfgs) { delete L(lbfgs); }
 
 int gmo_lbfgs_set_weight_buffers(uintptr_t lbfgs, const uintptr_t *buffers, int n)
 {
+    if (!lbfgs) return fail(Errorf("object handle is nil"));
     Error e = L(lbfgs)->SetWeightBuffers(pointers(buffers, n));
     return e.empty() ? ok() : fail(e);
 }
 
 int gmo_lbfgs_step(uintptr_t lbfgs, const uintptr_t *gradient_buffers, int n, float current_loss)
 {
+    if (!lbfgs) return fail(Errorf("object handle is nil"));
     Error e = L(lbfgs)->Step(pointers(gradient_buffers, n), current_loss);
     return e.empty() ? ok() : fail(e);
 }
 
 void gmo_lbfgs_set_command_pool(uintptr_t lbfgs, uintptr_t pool)
 {
+    if (!lbfgs) return;
     L(lbfgs)->SetCommandPool(reinterpret_cast<Pointer>(pool));
 }
 
-int gmo_lbfgs_uses_pooling(uintptr_t lbfgs) { return L(lbfgs)->usePooling ? 1 : 0; }
-uint64_t gmo_lbfgs_get_step(uintptr_t lbfgs) { return L(lbfgs)->GetStep(); }
+int gmo_lbfgs_uses_pooling(uintptr_t lbfgs) {
+    if (!lbfgs) return fail(Errorf("object handle is nil")); return L(lbfgs)->usePooling ? 1 : 0; }
+uint64_t gmo_lbfgs_get_step(uintptr_t lbfgs) {
+    if (!lbfgs) { fail(Errorf("object handle is nil")); return 0; } return L(lbfgs)->GetStep(); }
 
 void gmo_lbfgs_get_stats(uintptr_t lbfgs, uint64_t *step, int *history_size, int *history_used, float *prev_loss)
 {
+    if (!lbfgs) return;
     auto stats = L(lbfgs)->GetStats();
     if (step) *step = std::get<uint64_t>(stats.at("step"));
     if (history_size) *history_size = (int)std::get<uint64_t>(stats.at("history_size"));
@@ -481,29 +505,35 @@ void gmo_lbfgs_get_stats(uintptr_t lbfgs, uint64_t *step, int *history_size, int
 
 void gmo_lbfgs_history(uintptr_t lbfgs, int *count, int *index, float *last_step_size)
 {
+    if (!lbfgs) return;
     if (count) *count = L(lbfgs)->historyCount;
     if (index) *index = L(lbfgs)->historyIndex;
     if (last_step_size) *last_step_size = L(lbfgs)->lastStepSize;
 }
 
-void gmo_lbfgs_cleanup(uintptr_t lbfgs) { L(lbfgs)->Cleanup(); }
+void gmo_lbfgs_cleanup(uintptr_t lbfgs) {
+    if (!lbfgs) return; L(lbfgs)->Cleanup(); }
 
 int gmo_lbfgs_update_learning_rate(uintptr_t lbfgs, float lr)
 {
+    if (!lbfgs) return fail(Errorf("object handle is nil"));
     Error e = L(lbfgs)->UpdateLearningRate(lr);
     return e.empty() ? ok() : fail(e);
 }
 
-void gmo_lbfgs_set_log_progress(uintptr_t lbfgs, int on) { L(lbfgs)->logProgress = on != 0; }
+void gmo_lbfgs_set_log_progress(uintptr_t lbfgs, int on) {
+    if (!lbfgs) return; L(lbfgs)->logProgress = on != 0; }
 
 int gmo_lbfgs_buffer_size(uintptr_t lbfgs, int index)
 {
+    if (!lbfgs) return fail(Errorf("object handle is nil"));
     auto *l = L(lbfgs);
     return index >= 0 && (size_t)index < l->bufferSizes.size() ? l->bufferSizes[index] : -1;
 }
 
 uintptr_t gmo_lbfgs_buffer(uintptr_t lbfgs, const char *which, int history, int index)
 {
+    if (!lbfgs) { fail(Errorf("object handle is nil")); return 0; }
     auto *l = L(lbfgs);
     const std::string w = which ? which : "";
     const bool h_ok = history >= 0 && history < l->config.HistorySize;
@@ -533,16 +563,23 @@ uintptr_t gmo_tensor_new(const int *shape, int ndims, int dtype, int device_type
     return reinterpret_cast<uintptr_t>(t);
 }
 
-uintptr_t gmo_tensor_retain(uintptr_t tensor) { return reinterpret_cast<uintptr_t>(T(tensor)->Retain()); }
-void gmo_tensor_release(uintptr_t tensor) { if (tensor) T(tensor)->Release(); }
+uintptr_t gmo_tensor_retain(uintptr_t tensor) {
+    if (!tensor) { fail(Errorf("object handle is nil")); return 0; } return reinterpret_cast<uintptr_t>(T(tensor)->Retain()); }
+void gmo_tensor_release(uintptr_t tensor) {
+    if (!tensor) return; if (tensor) T(tensor)->Release(); }
 void gmo_tensor_free(uintptr_t tensor) { delete T(tensor); }
-uintptr_t gmo_tensor_buffer(uintptr_t tensor) { return reinterpret_cast<uintptr_t>(T(tensor)->MetalBuffer()); }
-int gmo_tensor_size(uintptr_t tensor) { return T(tensor)->Size(); }
-int gmo_tensor_ref_count(uintptr_t tensor) { return T(tensor)->RefCount(); }
-int gmo_tensor_dtype(uintptr_t tensor) { return (int)T(tensor)->DType(); }
+uintptr_t gmo_tensor_buffer(uintptr_t tensor) {
+    if (!tensor) { fail(Errorf("object handle is nil")); return 0; } return reinterpret_cast<uintptr_t>(T(tensor)->MetalBuffer()); }
+int gmo_tensor_size(uintptr_t tensor) {
+    if (!tensor) return fail(Errorf("object handle is nil")); return T(tensor)->Size(); }
+int gmo_tensor_ref_count(uintptr_t tensor) {
+    if (!tensor) return fail(Errorf("object handle is nil")); return T(tensor)->RefCount(); }
+int gmo_tensor_dtype(uintptr_t tensor) {
+    if (!tensor) return fail(Errorf("object handle is nil")); return (int)T(tensor)->DType(); }
 
 uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype)
 {
+    if (!tensor) { fail(Errorf("object handle is nil")); return 0; }
     auto [t, err] = T(tensor)->ConvertTo((memory::DataType)dtype);
     if (!err.empty()) {
         fail(err);
@@ -554,12 +591,14 @@ uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype)
 
 int gmo_tensor_copy_float32_data(uintptr_t tensor, const float *data, int n)
 {
+    if (!tensor) return fail(Errorf("object handle is nil"));
     Error e = T(tensor)->CopyFloat32Data(std::vector<float>(data, data + (n > 0 ? n : 0)));
     return e.empty() ? ok() : fail(e);
 }
 
 int gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity)
 {
+    if (!tensor) return fail(Errorf("object handle is nil"));
     auto [data, err] = T(tensor)->ToFloat32Slice();
     if (!err.empty()) return fail(err);
     if ((int)data.size() > capacity) return fail(Errorf("output holds %d elements, tensor has %d", capacity, (int)data.size()));
@@ -570,6 +609,7 @@ int gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity)
 
 int gmo_tensor_copy_from(uintptr_t dst, uintptr_t src)
 {
+    if (!dst) return fail(Errorf("object handle is nil"));
     Error e = T(dst)->CopyFrom(T(src));
     return e.empty() ? ok() : fail(e);
 }
@@ -582,7 +622,7 @@ int gmo_calculate_size(const int *shape, int ndims, int dtype)
 int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *weight_tensors, int num_weights,
                                                 const uintptr_t *gradient_tensors, int num_gradients)
 {
-    std::vector<memory::Tensor *> w, g;
+    std::vector<memory::Tensor *> w, g;     // a nil optimizer is the engine's own error case
     for (int k = 0; k < num_weights; k++) w.push_back(T(weight_tensors[k]));
     for (int k = 0; k < num_gradients; k++) g.push_back(T(gradient_tensors[k]));
     static const char *names[] = {"SGD", "Adam", "RMSProp", "AdaGrad", "AdaDelta", "Nadam"};
@@ -616,22 +656,26 @@ void gmo_scheduler_free(uintptr_t scheduler) { delete reinterpret_cast<Scheduler
 
 double gmo_scheduler_get_lr(uintptr_t scheduler, int epoch, int step, double base_lr)
 {
+    if (!scheduler) return std::nan("");
     return reinterpret_cast<SchedulerHandle *>(scheduler)->s->GetLR(epoch, step, base_lr);
 }
 
 double gmo_scheduler_plateau_step(uintptr_t scheduler, double metric, double current_lr)
 {
+    if (!scheduler) return std::nan("");
     auto *h = reinterpret_cast<SchedulerHandle *>(scheduler);
     if (h->kind != 3) return std::nan("");
     return static_cast<training::ReduceLROnPlateauScheduler *>(h->s.get())->Step(metric, current_lr);
 }
 
-const char *gmo_scheduler_name(uintptr_t scheduler) { return reinterpret_cast<SchedulerHandle *>(scheduler)->name.c_str(); }
+const char *gmo_scheduler_name(uintptr_t scheduler) {
+    if (!scheduler) { fail(Errorf("object handle is nil")); return ""; } return reinterpret_cast<SchedulerHandle *>(scheduler)->name.c_str(); }
 
 double gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, int step, double base_lr)
 {
+    if (!scheduler) return std::nan("");
     const double lr = gmo_scheduler_get_lr(scheduler, epoch, step, base_lr);
-    H(opt)->opt->UpdateLearningRate((float)lr);
+    if (opt) H(opt)->opt->UpdateLearningRate((float)lr);
     return lr;
 }
 

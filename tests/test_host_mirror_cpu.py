@@ -308,3 +308,28 @@ def test_lbfgs_default_config_and_constructor_errors(mm):
     else:
         opt.Cleanup()
         opt.free()
+
+
+def test_nil_object_handles_are_errors_not_crashes():
+    import ctypes
+    assert lib.gmo_step(0, None, 0) == -1 and lib.gmo_last_error() == b"object handle is nil"
+    assert lib.gmo_set_weight_buffers(0, None, 0) == -1
+    assert lib.gmo_get_step_count(0) == 0
+    assert lib.gmo_get_state_json(0) is None
+    assert lib.gmo_load_state_json(0, b"{}") == -1
+    assert math.isnan(lib.gmo_get_field(0, b"LearningRate"))
+    assert lib.gmo_state_buffer(0, b"momentum", 0) == 0
+    lib.gmo_cleanup(0)
+    lib.gmo_update_learning_rate(0, 0.1)
+    lib.gmo_optimizer_free(0)
+    assert lib.gmo_lbfgs_step(0, None, 0, 1.0) == -1
+    assert lib.gmo_lbfgs_get_step(0) == 0
+    lib.gmo_lbfgs_cleanup(0)
+    lib.gmo_lbfgs_free(0)
+    assert lib.gmo_tensor_size(0) == -1 and lib.gmo_tensor_buffer(0) == 0
+    assert lib.gmo_tensor_copy_from(0, 0) == -1
+    lib.gmo_tensor_release(0)
+    assert math.isnan(lib.gmo_scheduler_get_lr(0, 1, 1, 0.1))
+    sched = lib.gmo_scheduler_new(0, 10, 0.5, 0.0, None)
+    assert lib.gmo_scheduler_apply(sched, 0, 10, 0, 0.1) == pytest.approx(0.05)     # no optimizer to fan out to
+    lib.gmo_scheduler_free(sched)
