@@ -80,6 +80,16 @@ def time_steps(dev, launch, steps, warmup):
     return wall_ms / steps, event_ms / steps
 
 
+def per_launch_times(dev, launch, steps):
+    """HIP-event time of each of `steps` launches taken one at a time: (median ms, min ms)."""
+    times = []
+    for _ in range(steps):
+        dev.lib.gm_timer_start(dev.handle)
+        launch()
+        times.append(dev.lib.gm_timer_stop(dev.handle))
+    return float(np.median(times)), float(min(times))
+
+
 def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_seconds=12.0):
     """The CPU oracle (a C port of the reference's update equations, OpenMP over elements) on
     this host, on the leading tensors of the same workload up to ~budget_params, for about
@@ -238,12 +248,31 @@ def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
                       "runs this step as a single-threaded CPU loop)"}
 
 
+def run_all(args):
+    """Every configuration as a child process (this process never touches the GPU)."""
+    import subprocess
+    results = {}
+    for name in sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS):
+        cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", str(args.steps),
+               "--warmup", str(args.warmup)]
+        if args.no_cpu_baseline:
+            cmd.append("--no-cpu-baseline")
+        print(f"running {name}", file=sys.stderr, flush=True)
+        out = subprocess.run(cmd, check=True, stdout=subprocess.PIPE, text=True).stdout
+        results[name] = json.loads(out.strip().splitlines()[-1])
+    headline = dict(results["c5"])
+    headline["configs"] = {k: v for k, v in results.items() if k != "c5"}
+    print(json.dumps(headline))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS))
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["all"],
+                    help="'all': every configuration in turn, each in a process of its own; the line printed "
+                         "is the headline configuration's with the others under 'configs'")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
     ap.add_argument("--history", type=int, default=0, help="L-BFGS workloads: history size (default 10)")
@@ -255,6 +284,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the optimizer step shards without communication, and this "
                  "build runs and reports a single MI355X (--gpus 1).")
+
+    if args.workload == "all":
+        return run_all(args)
 
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -310,6 +342,7 @@ def main():
             raise RuntimeError(f"{rule} step failed rc={rc}: {lib.gm_last_error().decode()}")
 
     wall_ms, event_ms = time_steps(dev, launch_fp32, args.steps, args.warmup)
+    median_ms, min_ms = per_launch_times(dev, launch_fp32, args.steps)
     bpp = BYTES_PER_PARAM[rule]
     achieved = params * bpp / (event_ms * 1e-3) / 1e9
 
@@ -338,7 +371,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": f"multi_tensor_update_kernel<{rule}>", "bytes_per_param": bpp,
-                     "kernel_ms": event_ms, "copy_kernel_gbs": copy_gbs,
+                     "kernel_ms": event_ms, "kernel_ms_median": median_ms, "kernel_ms_min": min_ms,
+                     "copy_kernel_gbs": copy_gbs,
                      "frac_of_copy_kernel": achieved / copy_gbs},
     }
 
