@@ -143,6 +143,7 @@ HOST_ABI = {
     "gmo_scheduler_plateau_step": (ctypes.c_double, [u, ctypes.c_double, ctypes.c_double]),
     "gmo_scheduler_name": (c_str, [u]),
     "gmo_scheduler_apply": (ctypes.c_double, [u, u, i, i, ctypes.c_double]),
+    "gmo_pow": (f, [f, f]),
     "gmo_extract_buffer_index": (i, [c_str]),
     "gmo_calculate_tensor_size": (i, [ip, i]),
 }

@@ -679,6 +679,8 @@ double gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, int st
     return lr;
 }
 
+float gmo_pow(float x, float y) { return optimizer::pow(x, y); }
+
 int gmo_extract_buffer_index(const char *name) { return extractBufferIndex(name ? name : ""); }
 
 int gmo_calculate_tensor_size(const int *dims, int ndims)

@@ -39,6 +39,15 @@ Error validateStateType(const std::string &optimizerType, const OptimizerState *
 }
 
 // optimizer/adam.go:142-148
+float pow(float x, float y)
+{
+    if (y == 0) return 1.0f;
+    if (y == 1) return x;
+    float result = 1.0f;
+    for (int i = 0; i < (int)y; i++) result *= x;
+    return result;
+}
+
 int calculateTensorSize(const std::vector<int> &shape)
 {
     int size = 1;

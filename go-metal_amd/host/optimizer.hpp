@@ -78,6 +78,11 @@ bool extractBoolParam(const std::map<std::string, ParamValue> &params, const std
 uint64_t extractUint64Param(const std::map<std::string, ParamValue> &params, const std::string &key,
                             uint64_t defaultValue);
 
+// optimizer/adam.go:236-251: x^y by repeated multiplication for small non-negative integer y
+// (a helper the Go package keeps and tests but does not call; bias corrections are formed
+// natively with powf).
+float pow(float x, float y);
+
 using Shapes = std::vector<std::vector<int>>;
 
 // ------------------------------------------------------------------ SGD (optimizer/sgd.go) ----

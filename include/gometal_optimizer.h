@@ -144,6 +144,7 @@ const char *gmo_scheduler_name(uintptr_t scheduler);                            
 double      gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, int step, double base_lr);
 
 /* helpers (interface.go:56-76, adam.go:142-148) */
+float gmo_pow(float x, float y);                           /* pow, optimizer/adam.go:236-251 */
 int gmo_extract_buffer_index(const char *name);
 int gmo_calculate_tensor_size(const int *dims, int ndims);
 

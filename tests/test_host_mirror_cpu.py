@@ -333,3 +333,9 @@ def test_nil_object_handles_are_errors_not_crashes():
     sched = lib.gmo_scheduler_new(0, 10, 0.5, 0.0, None)
     assert lib.gmo_scheduler_apply(sched, 0, 10, 0, 0.1) == pytest.approx(0.05)     # no optimizer to fan out to
     lib.gmo_scheduler_free(sched)
+
+
+@pytest.mark.parametrize("x,y,expected", [(5.0, 0.0, 1.0), (5.0, 1.0, 5.0), (3.0, 2.0, 9.0), (2.0, 3.0, 8.0),
+                                          (-2.0, 2.0, 4.0), (1.5, 2.0, 2.25)])
+def test_pow_helper(x, y, expected):                        # adam_test.go:282-308
+    assert lib.gmo_pow(x, y) == expected
