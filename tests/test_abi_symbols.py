@@ -91,3 +91,27 @@ def test_host_scalars_match_oracle():
         bc1, bc2 = o.bias_corrections(0.9, 0.999, t)
         assert np.float32(a.value) == bc1 and np.float32(b.value) == bc2, t
         assert np.float32(lib.gm_nadam_mu_next(0.9, t)) == o.nadam_mu_next(0.9, t), t
+
+
+def test_headers_are_valid_c11(tmp_path):
+    """cgo compiles the preamble as C: both headers must parse with a C compiler, warnings as errors."""
+    import subprocess
+    src = tmp_path / "abi_check.c"
+    src.write_text('#include "gometal_hip.h"\n#include "gometal_optimizer.h"\n'
+                   "uintptr_t (*const probe_a)(void) = create_metal_device;\n"
+                   "int (*const probe_b)(uintptr_t, const uintptr_t *, int) = gmo_step;\n"
+                   "int main(void) { return 0; }\n")
+    subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only",
+                           "-I", os.path.join(ROOT, "include"), str(src)])
+
+
+def test_lbfgs_nil_device_and_history_checks_need_no_gpu():
+    pkg = load_package()
+    lib = pkg.load_library()
+    one = pkg.handle_array([0x1000])
+    size = pkg.int_array([64])
+    step = ctypes.c_float(-1.0)
+    args = (one, one, one, one, one, one, one, 0x1000, 1, size, 1, 0, 0, 1.0, 1e-4, 0.9, 20, 0.0, 0.0)
+    assert lib.execute_lbfgs_step_mpsgraph(0, *args, ctypes.byref(step)) == -1      # bridge_optimizer.m:1005-1009
+    assert lib.execute_lbfgs_step_mpsgraph_pooled(0, *args, 0x2000, ctypes.byref(step)) == -1
+    assert step.value == -1.0
