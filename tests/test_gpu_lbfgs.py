@@ -273,3 +273,72 @@ def test_c3_size_list_full_recursion(dev):
         assert_same_state(run.download(), ref, "c3")
     finally:
         run.free()
+
+
+def test_c4_size_list_two_valid_pairs(dev):
+    # 125M parameters in 60 tensors: three tree levels per dot product, every pass at scale
+    from workloads import amp_125m_sizes
+    sizes, m = amp_125m_sizes(), 2
+    rng = np.random.default_rng(125)
+    r = lambda k, s: rng.standard_normal(k, dtype=F) * F(s)
+    st = {"w": [r(k, 0.5) for k in sizes], "old_g": [r(k, 1e-2) for k in sizes],
+          "dir": [np.zeros(k, F) for k in sizes],
+          "s": [[r(k, 1e-2) for k in sizes] for _ in range(m)],
+          "y": [[r(k, 1e-2) for k in sizes] for _ in range(m)],
+          "rho": np.asarray([3e-4, -2e-4], dtype=F), "alpha": np.zeros(m, F)}
+    g = [r(k, 1e-2) for k in sizes]
+    run = LbfgsGpu(dev, st)
+    try:
+        run.step(g, 2, 0, 0.5)
+        print("oracle step over 125M parameters", flush=True)
+        assert oracle().lbfgs_step(st, g, m, 2, 0, 0.5, TREE)[0] == 0       # st is the reference from here on
+        assert_same_state(run.download(), st, "c4")
+        assert st["alpha"].all()
+    finally:
+        run.free()
+
+
+def test_c5_size_dot_and_plain_step(dev):
+    # 1,012,301,824 parameters in 400 tensors, data generated on the device: the dot product
+    # against the oracle's tree (four levels), and the step with no valid pair against its closed form
+    from workloads import transformer_block_sizes
+    sizes = transformer_block_sizes()
+    n, lib, D = len(sizes), dev.lib, dev.handle
+    lists = {}
+    for name, seed, std in (("w", 1, 0.02), ("g", 2, 1e-2), ("old_g", 3, 1e-2), ("dir", 4, 1.0), ("s", 5, 1e-2),
+                            ("y", 6, 1e-2)):
+        lists[name] = [dev.alloc(4 * k) for k in sizes]
+        for i, k in enumerate(sizes):
+            assert lib.gm_fill_normal_f32(D, lists[name][i], k, seed * 100000 + i, 0.0, std) == 0
+    rho, alpha = dev.from_numpy(np.zeros(1, F)), dev.from_numpy(np.zeros(1, F))
+    arr, bs = pkg.handle_array, pkg.int_array([4 * k for k in sizes])
+    try:
+        out = ctypes.c_float()
+        print("dot product over 1.012B parameters", flush=True)
+        assert lib.gm_lbfgs_dot(D, arr(lists["s"]), arr(lists["g"]), n, bs, ctypes.byref(out)) == 0
+        a = [dev.to_numpy(h, k) for h, k in zip(lists["s"], sizes)]
+        b = [dev.to_numpy(h, k) for h, k in zip(lists["g"], sizes)]
+        print("oracle dot product", flush=True)
+        assert F(out.value).view(np.uint32) == oracle().lbfgs_dot(a, b, TREE).view(np.uint32)
+        del a
+        w0 = [dev.to_numpy(lists["w"][i], sizes[i]) for i in (0, 2, 33, 399)]
+        step = ctypes.c_float()
+        # history_count 1 with rho = 0: update from the gradient, then the curvature pass
+        assert lib.execute_lbfgs_step_mpsgraph(D, arr(lists["w"]), arr(lists["g"]), arr(lists["old_g"]),
+                                               arr(lists["dir"]), arr(lists["s"]), arr(lists["y"]), arr([rho]),
+                                               alpha, n, bs, 1, 1, 0, 0.25, 1e-4, 0.9, 20, 0.0, 0.0,
+                                               ctypes.byref(step)) == 0
+        for j, i in enumerate((0, 2, 33, 399)):
+            k = sizes[i]
+            assert same_bits(dev.to_numpy(lists["w"][i], k), w0[j] + F(0.25) * b[i]), i
+            assert same_bits(dev.to_numpy(lists["dir"][i], k), b[i]), i
+            assert same_bits(dev.to_numpy(lists["old_g"][i], k), b[i]), i
+            assert same_bits(dev.to_numpy(lists["s"][i], k), F(0.25) * b[i]), i
+            assert not dev.to_numpy(lists["y"][i], k).any(), i
+        assert dev.to_numpy(rho, 1)[0] == 0.0 and dev.to_numpy(alpha, 1)[0] == 0.0
+    finally:
+        for hs in lists.values():
+            for h in hs:
+                dev.free(h)
+        dev.free(rho)
+        dev.free(alpha)
