@@ -62,6 +62,10 @@ ABI = {
     "gm_amp_state_destroy": (None, [u]),
     "gm_amp_state_get": (i, [u, fp, ip]),
     "gm_amp_state_set": (i, [u, f, i]),
+    "gm_amp_state_query": (i, [u, fp, ip, ip, ip]),
+    "gm_amp_state_set_step_count": (i, [u, i]),
+    "gm_amp_state_max_in_flight": (i, [u]),
+    "execute_adam_amp_step_async": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, u]),
     "execute_adam_amp_step": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, i, u, ip, fp, ip]),
     "gm_timer_start": (i, [u]),
     "gm_timer_stop": (f, [u]),
@@ -106,6 +110,8 @@ HOST_ABI = {
     "gmo_set_log_progress": (None, [u, i]),
     "gmo_enable_mixed_precision": (i, [u, f, f, f, i]),
     "gmo_step_amp": (i, [u, up, up, i, ip]),
+    "gmo_step_amp_async": (i, [u, up, up, i]),
+    "gmo_sync_amp": (i, [u, ctypes.POINTER(ctypes.c_uint64)]),
     "gmo_loss_scale": (f, [u]),
     "gmo_growth_tracker": (i, [u]),
     "gmo_lbfgs_default_config": (None, [ip, fp, ip, fp, fp, fp]),
@@ -357,6 +363,15 @@ class HostOptimizer:
         rc = self.lib.gmo_step_amp(self.handle, handle_array(gradient16_buffers), handle_array(weight16_buffers),
                                    len(gradient16_buffers), ctypes.byref(skipped))
         return bool(skipped.value), self._err(rc)
+
+    def StepAMPAsync(self, gradient16_buffers, weight16_buffers=None):
+        return self._err(self.lib.gmo_step_amp_async(self.handle, handle_array(gradient16_buffers),
+                                                     handle_array(weight16_buffers), len(gradient16_buffers)))
+
+    def SyncAMP(self):
+        skipped = ctypes.c_uint64(0)
+        rc = self.lib.gmo_sync_amp(self.handle, ctypes.byref(skipped))
+        return skipped.value, self._err(rc)
 
     def EnableMixedPrecision(self, initial_scale=65536.0, growth_factor=2.0, backoff_factor=0.5, growth_interval=2000):
         return self._err(self.lib.gmo_enable_mixed_precision(self.handle, initial_scale, growth_factor,

@@ -354,12 +354,25 @@ multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, 
 struct AmpDeviceState {
     float scale;
     int growth_tracker;
-    int found_inf;          // set by the check kernel, consumed and cleared by the update kernel
-    unsigned int reserved;
+    int found_inf;          // set by the check kernel, consumed and cleared by the epilogue
+    int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
     int last_skipped;
     float growth_factor;
     float backoff_factor;
     int growth_interval;
+    int skipped_steps;      // steps dropped so far
+    int pad;
+};
+
+// Bias corrections for the asynchronous step.  The host does not know how many of the steps
+// still in flight were applied, so it sends the corrections (glibc powf, like every other
+// step) for each step count that is possible and the kernel picks by the device's count.
+constexpr int kAmpMaxInFlight = 8;
+struct AmpBiasTable {
+    int base;               // step count of entry 0 minus one: entry j is for t = base + 1 + j
+    int count;              // 1: use entry 0 whatever the device's count (synchronous step)
+    float bc1[kAmpMaxInFlight];
+    float bc2[kAmpMaxInFlight];
 };
 
 // Phase A: OR over every fp16 gradient element of "exponent field all ones"
@@ -414,10 +427,14 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__re
 template <int VEC, bool NT>
 __global__ void __launch_bounds__(kBlock)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
-                       const AmpDeviceState *__restrict__ state)
+                       const AmpDeviceState *__restrict__ state, AmpBiasTable bias)
 {
     if (state->found_inf) return;
     const float inv_scale = 1.0f / state->scale;
+    int pick = bias.count > 1 ? state->applied_steps - bias.base : 0;
+    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
+    prm.bc1 = bias.bc1[pick];
+    prm.bc2 = bias.bc2[pick];
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
     update_slice<AdamRule, VEC, NT, true>(ch, slice_shift, prm, inv_scale);
 }
@@ -426,26 +443,29 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
 // loss-scale state machine and re-arms the flag.  A separate launch rather
 // than a last-workgroup ticket: a single counter bumped by every workgroup of
 // a 250k-workgroup grid serialises in the memory-side atomic unit.
-__global__ void amp_finalize_kernel(AmpDeviceState *state)
+__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    const int found = state->found_inf;
-    float s = state->scale;
-    int tracker = state->growth_tracker;
+    AmpDeviceState st = *state;
+    const int found = st.found_inf;
     if (found) {
-        s = s * state->backoff_factor;
-        tracker = 0;
+        st.scale = st.scale * st.backoff_factor;
+        st.growth_tracker = 0;
+        st.skipped_steps += 1;
     } else {
-        tracker += 1;
-        if (tracker == state->growth_interval) {
-            s = s * state->growth_factor;
-            tracker = 0;
+        st.applied_steps += 1;
+        st.growth_tracker += 1;
+        if (st.growth_tracker == st.growth_interval) {
+            st.scale = st.scale * st.growth_factor;
+            st.growth_tracker = 0;
         }
     }
-    state->scale = s;
-    state->growth_tracker = tracker;
-    state->last_skipped = found ? 1 : 0;
-    state->found_inf = 0;
+    st.last_skipped = found ? 1 : 0;
+    st.found_inf = 0;
+    *state = st;
+    // The post-state also goes straight into pinned host memory: the host reads it once the
+    // stream (or the event recorded after this launch) has completed, without a copy launch.
+    if (host_mirror) *host_mirror = st;
 }
 
 // ----------------------------------------------------------- host helpers ----
@@ -812,7 +832,13 @@ struct AmpState {
     uint64_t magic;
     Context *ctx;
     AmpDeviceState *d_state;
-    AmpDeviceState *h_pinned;
+    AmpDeviceState *h_pinned;            // kAmpMaxInFlight + 1 slots: [0] synchronous read-backs, [1..] the ring
+    hipEvent_t ring_event[kAmpMaxInFlight];
+    // asynchronous steps: issue numbers count execute_adam_amp_step_async calls
+    uint64_t issued;                     // steps issued so far
+    uint64_t confirmed_issue;            // newest step whose post-state the host has seen
+    int confirmed_applied;               // the device's applied_steps after that step
+    int max_in_flight;                   // deepest run-ahead seen (diagnostics)
 };
 static const uint64_t kAmpMagic = 0x676D5F616D705F73ull;   // "gm_amp_s"
 
@@ -830,11 +856,50 @@ static bool amp_upload(AmpState *s)
            hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize");
 }
 
+// Waits for everything on the stream and reads the state back: afterwards no step is in flight.
 static bool amp_download(AmpState *s)
 {
-    return hip_ok(hipMemcpyAsync(s->h_pinned, s->d_state, sizeof(AmpDeviceState),
-                                 hipMemcpyDeviceToHost, s->ctx->stream), "amp state download") &&
-           hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize");
+    if (!hip_ok(hipMemcpyAsync(s->h_pinned, s->d_state, sizeof(AmpDeviceState),
+                               hipMemcpyDeviceToHost, s->ctx->stream), "amp state download") ||
+        !hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize"))
+        return false;
+    s->confirmed_issue = s->issued;
+    s->confirmed_applied = s->h_pinned->applied_steps;
+    return true;
+}
+
+// Takes note of the asynchronous steps that have finished since the last look.  With
+// must_free_slot, blocks until at most kAmpMaxInFlight - 2 steps are unconfirmed, so that the
+// next step's bias table and ring slot are available.
+static bool amp_poll(AmpState *s, bool must_free_slot)
+{
+    for (;;) {
+        while (s->confirmed_issue < s->issued) {
+            const uint64_t next = s->confirmed_issue + 1;
+            const hipError_t q = hipEventQuery(s->ring_event[next % kAmpMaxInFlight]);
+            if (q == hipErrorNotReady) {
+                (void)hipGetLastError();     // "not ready" is an answer, not a failure to report later
+                break;
+            }
+            if (!hip_ok(q, "hipEventQuery")) return false;
+            s->confirmed_issue = next;
+            s->confirmed_applied = s->h_pinned[1 + next % kAmpMaxInFlight].applied_steps;
+        }
+        if (!must_free_slot || s->issued - s->confirmed_issue <= (uint64_t)kAmpMaxInFlight - 2) return true;
+        const uint64_t oldest = s->confirmed_issue + 1;
+        if (!hip_ok(hipEventSynchronize(s->ring_event[oldest % kAmpMaxInFlight]), "hipEventSynchronize"))
+            return false;
+    }
+}
+
+static void amp_free(AmpState *s)
+{
+    if (s->d_state) (void)hipFree(s->d_state);
+    if (s->h_pinned) (void)hipHostFree(s->h_pinned);
+    for (hipEvent_t e : s->ring_event)
+        if (e) (void)hipEventDestroy(e);
+    s->magic = 0;
+    delete s;
 }
 
 uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_factor,
@@ -844,20 +909,25 @@ uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_f
     if (device == 0) return 0;
     Context *ctx = resolve_device(device);
     if (!ctx || !make_current(ctx)) return 0;
-    auto *s = new AmpState{kAmpMagic, ctx, nullptr, nullptr};
-    if (!hip_ok(hipMalloc(&s->d_state, sizeof(AmpDeviceState)), "hipMalloc(amp state)") ||
-        !hip_ok(hipHostMalloc(&s->h_pinned, sizeof(AmpDeviceState), hipHostMallocDefault),
-                "hipHostMalloc(amp state)")) {
-        if (s->d_state) (void)hipFree(s->d_state);
-        delete s;
-        return 0;
+    auto *s = new AmpState{};
+    s->magic = kAmpMagic;
+    s->ctx = ctx;
+    bool ok = hip_ok(hipMalloc(&s->d_state, sizeof(AmpDeviceState)), "hipMalloc(amp state)") &&
+              hip_ok(hipHostMalloc(&s->h_pinned, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState),
+                                   hipHostMallocDefault), "hipHostMalloc(amp state)");
+    for (int k = 0; ok && k < kAmpMaxInFlight; k++)
+        ok = hip_ok(hipEventCreateWithFlags(&s->ring_event[k], hipEventDisableTiming), "hipEventCreate");
+    if (ok) {
+        std::memset(s->h_pinned, 0, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState));
+        s->h_pinned->scale = init_scale;
+        s->h_pinned->growth_factor = growth_factor;
+        s->h_pinned->backoff_factor = backoff_factor;
+        s->h_pinned->growth_interval = growth_interval;
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        ok = amp_upload(s);
     }
-    *s->h_pinned = AmpDeviceState{init_scale, 0, 0, 0u, 0, growth_factor, backoff_factor, growth_interval};
-    std::lock_guard<std::mutex> lk(ctx->mu);
-    if (!amp_upload(s)) {
-        (void)hipFree(s->d_state);
-        (void)hipHostFree(s->h_pinned);
-        delete s;
+    if (!ok) {
+        amp_free(s);
         return 0;
     }
     return reinterpret_cast<uintptr_t>(s);
@@ -868,13 +938,17 @@ void gm_amp_state_destroy(uintptr_t amp_state)
     AmpState *s = amp_from_handle(amp_state);
     if (!s) return;
     make_current(s->ctx);
-    s->magic = 0;
-    (void)hipFree(s->d_state);
-    (void)hipHostFree(s->h_pinned);
-    delete s;
+    (void)hipStreamSynchronize(s->ctx->stream);     // ring copies may still be in flight
+    amp_free(s);
 }
 
 int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker)
+{
+    return gm_amp_state_query(amp_state, scale, growth_tracker, nullptr, nullptr);
+}
+
+int gm_amp_state_query(uintptr_t amp_state, float *scale, int *growth_tracker, int *applied_steps,
+                       int *skipped_steps)
 {
     AmpState *s = amp_from_handle(amp_state);
     if (!s) return -16;
@@ -883,7 +957,15 @@ int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker)
     if (!amp_download(s)) return -6;
     if (scale) *scale = s->h_pinned->scale;
     if (growth_tracker) *growth_tracker = s->h_pinned->growth_tracker;
+    if (applied_steps) *applied_steps = s->h_pinned->applied_steps;
+    if (skipped_steps) *skipped_steps = s->h_pinned->skipped_steps;
     return 0;
+}
+
+int gm_amp_state_max_in_flight(uintptr_t amp_state)
+{
+    AmpState *s = amp_from_handle(amp_state);
+    return s ? s->max_in_flight : -16;
 }
 
 int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
@@ -898,17 +980,28 @@ int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
     return amp_upload(s) ? 0 : -6;
 }
 
-int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
-                          uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
-                          uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
-                          int num_weights, int *buffer_sizes, float learning_rate, float beta1,
-                          float beta2, float epsilon, float weight_decay, int step_count,
-                          uintptr_t amp_state, int *skipped, float *scale_out,
-                          int *growth_tracker_out)
+int gm_amp_state_set_step_count(uintptr_t amp_state, int applied_steps)
 {
-    if (device == 0) return -1;
-    AmpState *amp = amp_from_handle(amp_state);
-    if (!amp) return -16;
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (applied_steps < 0) return -5;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    s->h_pinned->applied_steps = applied_steps;
+    if (!amp_upload(s)) return -6;
+    s->confirmed_applied = applied_steps;
+    return 0;
+}
+
+// Plan, parameters and the three launches shared by the synchronous and the asynchronous step.
+static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffers,
+                       uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                       uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
+                       int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
+                       float weight_decay, int step_count, bool async, AmpDeviceState *host_mirror,
+                       Launch &l, std::unique_lock<std::mutex> &lock)
+{
     PlanRequest req{};
     req.kind = kRuleAdamAMP;
     req.num_tensors = num_weights;
@@ -921,9 +1014,11 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
     req.required_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0) | (1u << kSlotState1);
     req.missing_code = -4;
     req.half_mask = (1u << kSlotGrad) | (1u << kSlotWeight16);
-    Launch l{};
-    std::unique_lock<std::mutex> lock;
     if (int rc = prepare(device, req, -6, l, lock)) return rc;
+    if (l.ctx != amp->ctx) {
+        set_error("the loss-scale state belongs to another device context");
+        return -16;
+    }
 
     StepParams p = zero_params();
     p.lr = learning_rate;
@@ -933,7 +1028,20 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
     p.one_minus_beta2 = 1.0f - beta2;
     p.eps = epsilon;
     p.weight_decay = weight_decay;
-    gm_bias_corrections(beta1, beta2, step_count, &p.bc1, &p.bc2);
+
+    AmpBiasTable bias{};
+    if (async) {
+        if (!amp_poll(amp, true)) return -6;
+        const int in_flight = (int)(amp->issued - amp->confirmed_issue);
+        if (in_flight > amp->max_in_flight) amp->max_in_flight = in_flight;
+        bias.base = amp->confirmed_applied;
+        bias.count = in_flight + 1;
+        for (int j = 0; j <= in_flight; j++)
+            gm_bias_corrections(beta1, beta2, amp->confirmed_applied + 1 + j, &bias.bc1[j], &bias.bc2[j]);
+    } else {
+        bias.count = 1;
+        gm_bias_corrections(beta1, beta2, step_count, &bias.bc1[0], &bias.bc2[0]);
+    }
 
     const uint32_t chunks = l.plan->num_chunks;
     hipStream_t st = l.ctx->stream;
@@ -944,18 +1052,66 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
         if (!launch_geometry(*l.plan, vec, grid, shift)) return -6;
         if (nt) amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
         else amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
-#define GM_LAUNCH_AMP(V, N) amp_adam_update_kernel<V, N><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, shift, p, amp->d_state)
+#define GM_LAUNCH_AMP(V, N) amp_adam_update_kernel<V, N><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, shift, p, amp->d_state, bias)
         if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true); else GM_LAUNCH_AMP(4, false); }
         else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true); else GM_LAUNCH_AMP(2, false); }
         else { if (nt) GM_LAUNCH_AMP(1, true); else GM_LAUNCH_AMP(1, false); }
 #undef GM_LAUNCH_AMP
     }
-    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state);
-    if (!hip_ok(hipGetLastError(), "mixed-precision kernel launch")) return -6;
-    if (!amp_download(amp)) return -6;
+    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror);
+    return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
+}
+
+int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
+                          uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                          uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                          int num_weights, int *buffer_sizes, float learning_rate, float beta1,
+                          float beta2, float epsilon, float weight_decay, int step_count,
+                          uintptr_t amp_state, int *skipped, float *scale_out,
+                          int *growth_tracker_out)
+{
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = amp_enqueue(device, amp, weight_buffers, gradient16_buffers, momentum_buffers,
+                             variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
+                             beta1, beta2, epsilon, weight_decay, step_count, false, amp->h_pinned, l, lock))
+        return rc;
+    if (!hip_ok(hipStreamSynchronize(l.ctx->stream), "hipStreamSynchronize")) return -6;
+    amp->confirmed_issue = amp->issued;
+    amp->confirmed_applied = amp->h_pinned->applied_steps;
     if (skipped) *skipped = amp->h_pinned->last_skipped;
     if (scale_out) *scale_out = amp->h_pinned->scale;
     if (growth_tracker_out) *growth_tracker_out = amp->h_pinned->growth_tracker;
+    return 0;
+}
+
+int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
+                                uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                                uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                                int num_weights, int *buffer_sizes, float learning_rate, float beta1,
+                                float beta2, float epsilon, float weight_decay, uintptr_t amp_state)
+{
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    // the post-state of this step goes into its ring slot; the event marks its arrival
+    const uint64_t issue = amp->issued + 1;
+    const int slot = (int)(issue % kAmpMaxInFlight);
+    if (int rc = amp_enqueue(device, amp, weight_buffers, gradient16_buffers, momentum_buffers,
+                             variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
+                             beta1, beta2, epsilon, weight_decay, 0, true, &amp->h_pinned[1 + slot], l, lock))
+        return rc;
+    if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
+        // the step itself is enqueued; resynchronise the bookkeeping with the device
+        (void)amp_download(amp);
+        return -6;
+    }
+    amp->issued = issue;
     return 0;
 }
 

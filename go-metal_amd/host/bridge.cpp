@@ -386,5 +386,28 @@ Error ExecuteAdamAMPStep(Pointer device, const std::vector<Pointer> &weightBuffe
     return "";
 }
 
+Error ExecuteAdamAMPStepAsync(Pointer device, const std::vector<Pointer> &weightBuffers,
+                              const std::vector<Pointer> &gradient16Buffers,
+                              const std::vector<Pointer> &momentumBuffers,
+                              const std::vector<Pointer> &varianceBuffers,
+                              const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes,
+                              float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
+                              Pointer ampState)
+{
+    const size_t n = weightBuffers.size();
+    if (n != gradient16Buffers.size() || n != momentumBuffers.size() || n != varianceBuffers.size() ||
+        n != bufferSizes.size() || (!weight16Buffers.empty() && weight16Buffers.size() != n))
+        return Errorf("all buffer arrays must have the same length");
+    if (n == 0) return Errorf("%s", kEmptyList);
+    auto w = handles(weightBuffers, n), g = handles(gradient16Buffers, n), m = handles(momentumBuffers, n),
+         v = handles(varianceBuffers, n), h = handles(weight16Buffers, n);
+    std::vector<int> sizes(bufferSizes);
+    int result = execute_adam_amp_step_async(H(device), w.data(), g.data(), m.data(), v.data(),
+                                             weight16Buffers.empty() ? nullptr : h.data(), (int)n, sizes.data(),
+                                             learningRate, beta1, beta2, epsilon, weightDecay, H(ampState));
+    if (result != 0) return Errorf("Adam mixed-precision step failed with error code: %d", result);
+    return "";
+}
+
 }  // namespace cgo_bridge
 }  // namespace gometal

@@ -109,5 +109,14 @@ Error ExecuteAdamAMPStep(Pointer device, const std::vector<Pointer> &weightBuffe
                          float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
                          int stepCount, Pointer ampState, bool *skipped, float *scale, int *growthTracker);
 
+// The same step without the read-back (execute_adam_amp_step_async).
+Error ExecuteAdamAMPStepAsync(Pointer device, const std::vector<Pointer> &weightBuffers,
+                              const std::vector<Pointer> &gradient16Buffers,
+                              const std::vector<Pointer> &momentumBuffers,
+                              const std::vector<Pointer> &varianceBuffers,
+                              const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes,
+                              float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
+                              Pointer ampState);
+
 }  // namespace cgo_bridge
 }  // namespace gometal

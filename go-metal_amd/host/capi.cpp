@@ -416,6 +416,22 @@ int gmo_step_amp(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintp
     return ok();
 }
 
+int gmo_step_amp_async(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n)
+{
+    auto *a = adam_of(opt);
+    if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
+    Error e = a->StepAMPAsync(pointers(gradient16_buffers, n), pointers(weight16_buffers, weight16_buffers ? n : 0));
+    return e.empty() ? ok() : fail(e);
+}
+
+int gmo_sync_amp(uintptr_t opt, uint64_t *skipped_steps)
+{
+    auto *a = adam_of(opt);
+    if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
+    Error e = a->SyncAMP(skipped_steps);
+    return e.empty() ? ok() : fail(e);
+}
+
 float gmo_loss_scale(uintptr_t opt)
 {
     if (!opt) return std::nanf("");

@@ -392,10 +392,19 @@ Error AdamOptimizerState::SetWeightBuffers(const std::vector<Pointer> &weightBuf
     return setWeights(WeightBuffers, weightBuffers);
 }
 
+uint64_t AdamOptimizerState::GetStepCount()
+{
+    if (ampPending > 0) (void)SyncAMP();     // pending asynchronous steps: the device holds the count
+    return StepCount;
+}
+
 Error AdamOptimizerState::Step(const std::vector<Pointer> &gradientBuffers)
 {
     if (Error e = checkGradients(gradientBuffers, WeightBuffers); !e.empty()) return e;
+    if (ampPending > 0)
+        if (Error e = SyncAMP(); !e.empty()) return e;
     StepCount++;
+    ampCountDirty = true;
     // As in adam.go:191-227 the pooled entry point is not used even when a pool is set.
     Error err = cgo_bridge::ExecuteAdamStepMPSGraph(device, WeightBuffers, gradientBuffers, MomentumBuffers,
                                                     VarianceBuffers, bufferSizes, LearningRate, Beta1, Beta2,
@@ -416,6 +425,41 @@ Error AdamOptimizerState::EnableMixedPrecision(float initialScale, float growthF
     if (ampState == nullptr) return Errorf("failed to create loss-scale state: %s", gm_last_error());
     LossScale = initialScale;
     GrowthTracker = 0;
+    ampPending = 0;
+    ampCountDirty = true;
+    return "";
+}
+
+Error AdamOptimizerState::SyncAMP(uint64_t *skippedSteps)
+{
+    if (ampState == nullptr) return Errorf("mixed precision is not enabled: call EnableMixedPrecision first");
+    int applied = 0, skipped = 0;
+    if (gm_amp_state_query(reinterpret_cast<uintptr_t>(ampState), &LossScale, &GrowthTracker, &applied, &skipped) != 0)
+        return Errorf("failed to read loss-scale state: %s", gm_last_error());
+    if (ampPending > 0) StepCount = (uint64_t)applied;     // the device counted the pending steps
+    ampPending = 0;
+    if (skippedSteps) *skippedSteps = (uint64_t)skipped;
+    return "";
+}
+
+Error AdamOptimizerState::StepAMPAsync(const std::vector<Pointer> &gradient16Buffers,
+                                       const std::vector<Pointer> &weight16Buffers)
+{
+    if (Error e = checkGradients(gradient16Buffers, WeightBuffers); !e.empty()) return e;
+    if (!weight16Buffers.empty() && weight16Buffers.size() != WeightBuffers.size())
+        return Errorf("fp16 weight buffers length (%d) doesn't match weight buffers length (%d)",
+                      (int)weight16Buffers.size(), (int)WeightBuffers.size());
+    if (ampState == nullptr) return Errorf("mixed precision is not enabled: call EnableMixedPrecision first");
+    if (ampCountDirty) {
+        if (gm_amp_state_set_step_count(reinterpret_cast<uintptr_t>(ampState), (int)StepCount) != 0)
+            return Errorf("failed to set the device step count: %s", gm_last_error());
+        ampCountDirty = false;
+    }
+    Error err = cgo_bridge::ExecuteAdamAMPStepAsync(device, WeightBuffers, gradient16Buffers, MomentumBuffers,
+                                                    VarianceBuffers, weight16Buffers, bufferSizes, LearningRate,
+                                                    Beta1, Beta2, Epsilon, WeightDecay, ampState);
+    if (!err.empty()) return Errorf("Adam mixed-precision step execution failed: %s", err.c_str());
+    ampPending++;
     return "";
 }
 
@@ -427,6 +471,13 @@ std::pair<bool, Error> AdamOptimizerState::StepAMP(const std::vector<Pointer> &g
         return {false, Errorf("fp16 weight buffers length (%d) doesn't match weight buffers length (%d)",
                               (int)weight16Buffers.size(), (int)WeightBuffers.size())};
     if (ampState == nullptr) return {false, Errorf("mixed precision is not enabled: call EnableMixedPrecision first")};
+    if (ampPending > 0)
+        if (Error e = SyncAMP(); !e.empty()) return {false, e};
+    if (ampCountDirty) {
+        if (gm_amp_state_set_step_count(reinterpret_cast<uintptr_t>(ampState), (int)StepCount) != 0)
+            return {false, Errorf("failed to set the device step count: %s", gm_last_error())};
+        ampCountDirty = false;
+    }
     bool skipped = false;
     // StepCount advances only when the step is applied: the bias corrections are taken at StepCount + 1.
     Error err = cgo_bridge::ExecuteAdamAMPStep(device, WeightBuffers, gradient16Buffers, MomentumBuffers,
@@ -465,6 +516,8 @@ void AdamOptimizerState::Cleanup()
 
 StateResult AdamOptimizerState::GetState()
 {
+    if (ampPending > 0)
+        if (Error e = SyncAMP(); !e.empty()) return {nullptr, e};
     auto st = std::make_unique<OptimizerState>();
     if (Error e = readBuffers(MomentumBuffers, bufferSizes, "momentum", "momentum", "momentum", st->StateData); !e.empty())
         return {nullptr, e};
@@ -484,6 +537,9 @@ StateResult AdamOptimizerState::GetState()
 Error AdamOptimizerState::LoadState(const OptimizerState *state)
 {
     if (Error e = validateStateType("Adam", state); !e.empty()) return e;
+    if (ampPending > 0)
+        if (Error e = SyncAMP(); !e.empty()) return e;
+    ampCountDirty = true;
     setFloat(state->Parameters, "learning_rate", LearningRate);
     setFloat(state->Parameters, "beta1", Beta1);
     setFloat(state->Parameters, "beta2", Beta2);

@@ -142,8 +142,8 @@ public:
     Error Step(const std::vector<Pointer> &gradientBuffers) override;
     std::pair<std::unique_ptr<OptimizerState>, Error> GetState() override;
     Error LoadState(const OptimizerState *state) override;
-    uint64_t GetStepCount() override { return StepCount; }   // additive: the Go type only has GetStep
-    uint64_t GetStep() { return StepCount; }
+    uint64_t GetStepCount() override;                         // additive: the Go type only has GetStep
+    uint64_t GetStep() { return GetStepCount(); }
     AdamStats GetStats();
     void UpdateLearningRate(float lr) override { LearningRate = lr; }
     Error SetWeightBuffers(const std::vector<Pointer> &weightBuffers) override;
@@ -159,7 +159,15 @@ public:
     // weight16Buffers may be empty (no fp16 weight copy).
     std::pair<bool, Error> StepAMP(const std::vector<Pointer> &gradient16Buffers,
                                    const std::vector<Pointer> &weight16Buffers);
-    float LossScale = 0.0f;     // as of the last StepAMP / EnableMixedPrecision / LoadState
+    // The same step without waiting for it: no result is returned, and up to 7 steps run ahead
+    // of the host.  StepCount, LossScale and GrowthTracker are brought up to date by SyncAMP
+    // (GetStepCount, GetState, LoadState, Step and StepAMP call it when steps are pending).
+    Error StepAMPAsync(const std::vector<Pointer> &gradient16Buffers,
+                       const std::vector<Pointer> &weight16Buffers);
+    // Waits for the pending steps; *skippedSteps (may be null) receives how many steps have
+    // been dropped since EnableMixedPrecision.
+    Error SyncAMP(uint64_t *skippedSteps = nullptr);
+    float LossScale = 0.0f;     // as of the last StepAMP / SyncAMP / EnableMixedPrecision / LoadState
     int GrowthTracker = 0;
 
     memory::MemoryManager *memoryManager = nullptr;
@@ -168,6 +176,8 @@ public:
     Pointer commandPool = nullptr;
     bool usePooling = false;
     Pointer ampState = nullptr;
+    int ampPending = 0;            // asynchronous steps issued since the last SyncAMP
+    bool ampCountDirty = false;    // StepCount changed on the host since the device last saw it
 };
 std::pair<std::unique_ptr<AdamOptimizerState>, Error> NewAdamOptimizer(const AdamConfig &config,
                                                                        const Shapes &weightShapes,

@@ -239,6 +239,17 @@ void gm_amp_state_destroy(uintptr_t amp_state);
 /* Reads / overwrites scale and the clean-step counter (checkpointing). */
 int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker);
 int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker);
+/* As gm_amp_state_get, plus the number of steps applied (the optimizer's StepCount as the
+ * device counts it: +1 per clean step) and dropped since creation / the last
+ * gm_amp_state_set_step_count.  Waits for every step in flight.  Pointers may be NULL. */
+int gm_amp_state_query(uintptr_t amp_state, float *scale, int *growth_tracker, int *applied_steps,
+                       int *skipped_steps);
+/* The largest number of asynchronous steps that were still unconfirmed when another one was
+ * issued (0 to 6): tells whether a caller actually ran ahead of the device.  -16: nil state. */
+int gm_amp_state_max_in_flight(uintptr_t amp_state);
+/* Sets the device's applied-step count (call when the optimizer's StepCount is set by other
+ * means: construction, LoadState).  -5: negative count. */
+int gm_amp_state_set_step_count(uintptr_t amp_state, int applied_steps);
 
 /* One mixed-precision Adam step over the whole tensor list.
  *   gradient16_buffers: fp16 gradients of the SCALED loss (read only)
@@ -262,6 +273,20 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
                           float beta2, float epsilon, float weight_decay, int step_count,
                           uintptr_t amp_state, int *skipped, float *scale_out,
                           int *growth_tracker_out);
+
+/* execute_adam_amp_step without the read-back: enqueues the step and returns.  The bias-correction
+ * step is taken from the device's own applied-step count (gm_amp_state_set_step_count, +1 per
+ * clean step), so a dropped step needs no host decision: the host sends the corrections for
+ * every count that the steps still in flight leave possible (at most 8) and the kernel picks.
+ * Up to 7 steps run ahead of the host; the call waits for the oldest one beyond that.
+ * Results and counters are read with gm_amp_state_query (which waits).  Buffers, arithmetic
+ * and results are exactly those of the synchronous step.  Codes as execute_adam_amp_step. */
+int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
+                                uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                                uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                                int num_weights, int *buffer_sizes, float learning_rate,
+                                float beta1, float beta2, float epsilon, float weight_decay,
+                                uintptr_t amp_state);
 
 /* The dot product of two tensor lists exactly as the L-BFGS step forms it (fp64 tree,
  * one rounding to fp32).  Synchronises.  Codes as execute_lbfgs_step_mpsgraph. */

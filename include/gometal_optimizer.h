@@ -84,6 +84,9 @@ int   gmo_enable_mixed_precision(uintptr_t adam, float initial_scale, float grow
                                  int growth_interval);
 int   gmo_step_amp(uintptr_t adam, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n,
                    int *skipped);
+int   gmo_step_amp_async(uintptr_t adam, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers,
+                         int n);                     /* StepAMPAsync: no wait, no result */
+int   gmo_sync_amp(uintptr_t adam, uint64_t *skipped_steps);   /* SyncAMP: waits, refreshes StepCount / scale */
 float gmo_loss_scale(uintptr_t adam);
 int   gmo_growth_tracker(uintptr_t adam);
 

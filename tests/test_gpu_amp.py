@@ -178,3 +178,64 @@ def test_amp_full_size(dev, name, sizes_fn, weight_decay):
         pair.compare("final")
     finally:
         pair.close()
+
+
+def test_async_steps_equal_the_synchronous_sequence(dev):
+    """execute_adam_amp_step_async in bursts the host does not wait for: the device picks the bias
+    corrections by its own applied-step count.  After every burst the counters, and every few bursts
+    all buffers, must equal the oracle's (which is what the synchronous step is held to)."""
+    pkg = load_package()
+    lib, D = dev.lib, dev.handle
+    rng = np.random.default_rng(0xA51)
+    sizes = [3_000_000, 4096, 2_000_000, 77, 1_500_000]
+    n, burst, bursts = len(sizes), 12, 24
+    amp_cfg = (1024.0, 2.0, 0.5, 7)                      # short growth interval: the scale moves often
+    w = [rng.normal(0, 0.02, s).astype(np.float32) for s in sizes]
+    pair = AmpPair(dev, w, dict(HYPER, weight_decay=1e-4), amp_cfg, nthreads=NTHREADS)
+    grads = [[rng.normal(0, 1e-3, s).astype(np.float32) for s in sizes] for _ in range(3)]
+    # one set of device gradient buffers per step of a burst, so that nothing is uploaded between steps
+    g16_dev = [[dev.alloc(2 * s) for s in sizes] for _ in range(burst)]
+    g16_arr = [pkg.handle_array(hs) for hs in g16_dev]
+    h = pair.h
+    assert lib.gm_amp_state_set_step_count(pair.amp, 0) == 0
+    try:
+        skipped_total = 0
+        for b in range(bursts):
+            # the oracle runs the burst first: it fixes the scale each step's gradients are made with
+            for j in range(burst):
+                scale = np.float32(pair.st.scale)
+                g16 = [(g * scale).astype(np.float16).view(np.uint16) for g in grads[(b + j) % 3]]
+                if rng.random() < 0.12:
+                    t = int(rng.integers(0, n))
+                    g16[t][int(rng.integers(0, sizes[t]))] = [0x7C00, 0xFC00, 0x7E00][(b + j) % 3]
+                for hd, g in zip(g16_dev[j], g16):
+                    dev.upload(hd, g)
+                skipped_total += oracle().adam_amp(pair.w, g16, pair.m, pair.v, pair.w16, state=pair.st,
+                                                   nthreads=NTHREADS, **h)
+            print(f"burst {b}: issuing {burst} steps", flush=True)
+            for j in range(burst):
+                rc = lib.execute_adam_amp_step_async(D, pair.c["w"], g16_arr[j], pair.c["m"], pair.c["v"],
+                                                     pair.c["w16"], n, pair.bs, h["lr"], h["beta1"], h["beta2"],
+                                                     h["eps"], h["weight_decay"], pair.amp)
+                assert rc == 0, (rc, lib.gm_last_error())
+            scale, tracker, applied, skipped = ctypes.c_float(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+            assert lib.gm_amp_state_query(pair.amp, ctypes.byref(scale), ctypes.byref(tracker),
+                                          ctypes.byref(applied), ctypes.byref(skipped)) == 0
+            assert (scale.value, tracker.value, applied.value, skipped.value) == \
+                (float(np.float32(pair.st.scale)), pair.st.growth_tracker, pair.st.step_count, skipped_total), b
+            if b % 6 == 5 or b == bursts - 1:
+                pair.compare(f"burst {b}")
+        assert 10 < skipped_total < burst * bursts - 50
+        # the host did run ahead: without it the bias table is never more than one entry long
+        assert lib.gm_amp_state_max_in_flight(pair.amp) >= 2
+        # a synchronous step continues from the same counters
+        scale = np.float32(pair.st.scale)
+        g16 = [(g * scale).astype(np.float16).view(np.uint16) for g in grads[0]]
+        pair.gpu_steps = pair.st.step_count
+        assert pair.step(g16) == 0
+        pair.compare("synchronous step after the bursts")
+    finally:
+        pair.close()
+        for hs in g16_dev:
+            for hd in hs:
+                dev.free(hd)

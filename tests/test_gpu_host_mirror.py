@@ -214,3 +214,78 @@ def test_step_amp_through_the_mirror(env):
     opt.free()
     for h in dw + dw16 + dg:
         dev.free(h)
+
+
+def test_step_amp_async_through_the_mirror(env):
+    """StepAMPAsync mixed with Step and StepAMP: the device keeps the step count while steps are
+    pending, and every host-side reader of StepCount catches up first."""
+    dev, mm = env
+    rng = np.random.default_rng(18)
+    sizes = [int(np.prod(s)) for s in SHAPES]
+    cfg, hyper = CASES[2][1], CASES[2][2]
+    opt = make(env, "adam", cfg)
+    assert opt.StepAMPAsync([0] * len(sizes)) == "mixed precision is not enabled: call EnableMixedPrecision first"
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    dw = [dev.from_numpy(a) for a in w]
+    dw16 = [dev.alloc(2 * n + 2, zero=True) for n in sizes]
+    dg32 = [dev.alloc(4 * n) for n in sizes]
+    dg = [dev.alloc(2 * n + 2) for n in sizes]
+    assert opt.SetWeightBuffers(dw) is None
+    ref = OracleRun("adam", hyper, w)
+    # two plain fp32 steps first: StepCount = 2 before mixed precision starts
+    for _ in range(2):
+        g = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
+        for h, a in zip(dg32, g):
+            dev.upload(h, a)
+        assert opt.Step(dg32) is None
+        ref.step(g)
+    assert opt.EnableMixedPrecision(4096.0, 2.0, 0.5, 2) is None
+    st = oracle().amp_state(4096.0, 2.0, 0.5, 2)
+    st.step_count = 2
+    m, v = ref.state["m"], ref.state["v"]
+    w16 = [np.zeros(n, np.uint16) for n in sizes]
+    skipped_want = 0
+    for k in range(7):
+        g16 = [(rng.normal(0, 1e-4, n) * st.scale).astype(np.float16).view(np.uint16) for n in sizes]
+        if k in (1, 4):
+            g16[2][7] = 0xFC00
+        for h, g in zip(dg, g16):
+            dev.upload(h, g)
+        assert opt.StepAMPAsync(dg, dw16) is None
+        skipped_want += oracle().adam_amp(ref.w, g16, m, v, w16, state=st, **hyper)
+    assert opt.GetStepCount() == st.step_count == 7          # 2 + 7 - 2 dropped; the call waits for the steps
+    skipped, err = opt.SyncAMP()
+    assert err is None and skipped == skipped_want == 2
+    assert dev.lib.gmo_loss_scale(opt.handle) == float(np.float32(st.scale))
+    assert dev.lib.gmo_growth_tracker(opt.handle) == st.growth_tracker
+    # a synchronous mixed-precision step and a plain step continue from there
+    g16 = [(rng.normal(0, 1e-4, n) * st.scale).astype(np.float16).view(np.uint16) for n in sizes]
+    for h, g in zip(dg, g16):
+        dev.upload(h, g)
+    skipped, err = opt.StepAMP(dg, dw16)
+    assert err is None and not skipped
+    oracle().adam_amp(ref.w, g16, m, v, w16, state=st, **hyper)
+    ref.step_count = st.step_count
+    g = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
+    for h, a in zip(dg32, g):
+        dev.upload(h, a)
+    assert opt.Step(dg32) is None
+    ref.step(g)
+    assert opt.GetStepCount() == ref.step_count == 9
+    # and one more asynchronous step after the plain one (the host pushes its count to the device)
+    st.step_count = 9
+    g16 = [(rng.normal(0, 1e-4, n) * st.scale).astype(np.float16).view(np.uint16) for n in sizes]
+    for h, gg in zip(dg, g16):
+        dev.upload(h, gg)
+    assert opt.StepAMPAsync(dg, dw16) is None
+    oracle().adam_amp(ref.w, g16, m, v, w16, state=st, **hyper)
+    text, err = opt.GetStateJSON()                            # catches up before reading
+    assert err is None and json.loads(text)["parameters"]["step_count"] == 10
+    for k, n in enumerate(sizes):
+        assert np.array_equal(dev.to_numpy(dw[k], n).view(np.uint32), ref.w[k].view(np.uint32)), k
+        assert np.array_equal(dev.to_numpy(dw16[k], n, np.uint16), w16[k]), k
+        assert np.array_equal(dev.to_numpy(opt.state_buffer("momentum", k), n).view(np.uint32), m[k].view(np.uint32))
+    opt.Cleanup()
+    opt.free()
+    for h in dw + dw16 + dg + dg32:
+        dev.free(h)
