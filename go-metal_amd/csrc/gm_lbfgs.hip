@@ -90,8 +90,7 @@ struct Plan {
     // scratch
     double *d_partial[2] = {nullptr, nullptr};
     LbScalars *d_scalars = nullptr;
-    int *d_valid = nullptr;
-    int *h_valid = nullptr;            // pinned
+    int *h_valid = nullptr;            // pinned host memory, written by the prologue kernel
     int valid_capacity = 0;
 
     ~Plan()
@@ -101,7 +100,6 @@ struct Plan {
         if (d_partial[0]) (void)hipFree(d_partial[0]);
         if (d_partial[1]) (void)hipFree(d_partial[1]);
         if (d_scalars) (void)hipFree(d_scalars);
-        if (d_valid) (void)hipFree(d_valid);
         if (h_valid) (void)hipHostFree(h_valid);
     }
 };
@@ -469,13 +467,10 @@ int stage_handles(Context *ctx, Plan &p, int n, int m, const uintptr_t *w, const
     }
     if (p.valid_capacity < m) {
         if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize")) return -8;
-        if (p.d_valid) (void)hipFree(p.d_valid);
         if (p.h_valid) (void)hipHostFree(p.h_valid);
-        p.d_valid = nullptr;
         p.h_valid = nullptr;
         p.valid_capacity = 0;
-        if (!hip_ok(hipMalloc(&p.d_valid, (size_t)m * sizeof(int)), "hipMalloc(lbfgs flags)") ||
-            !hip_ok(hipHostMalloc(&p.h_valid, (size_t)m * sizeof(int), hipHostMallocDefault),
+        if (!hip_ok(hipHostMalloc(&p.h_valid, (size_t)m * sizeof(int), hipHostMallocDefault),
                     "hipHostMalloc(lbfgs flags)"))
             return -8;
         p.valid_capacity = m;
@@ -597,10 +592,9 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uin
     // which pairs take part: one small read-back per step
     std::vector<int> valid;
     if (history_count > 0) {
-        lbfgs_prologue_kernel<<<1, 64, 0, stream>>>(r.rho, m, history_count, history_index, alpha, p.d_valid);
+        // the flags are written straight into pinned host memory: one wait, no copy launch
+        lbfgs_prologue_kernel<<<1, 64, 0, stream>>>(r.rho, m, history_count, history_index, alpha, p.h_valid);
         if (!hip_ok(hipGetLastError(), "L-BFGS prologue launch") ||
-            !hip_ok(hipMemcpyAsync(p.h_valid, p.d_valid, (size_t)history_count * sizeof(int),
-                                   hipMemcpyDeviceToHost, stream), "read L-BFGS pair flags") ||
             !hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize"))
             return -8;
         for (int j = 0; j < history_count; j++)
