@@ -90,6 +90,7 @@ struct Plan {
     // scratch
     double *d_partial[2] = {nullptr, nullptr};
     LbScalars *d_scalars = nullptr;
+    unsigned int *d_ticket = nullptr;  // workgroup counter of the fused reduction, zero between launches
     int *h_valid = nullptr;            // pinned host memory, written by the prologue kernel
     int valid_capacity = 0;
 
@@ -100,6 +101,7 @@ struct Plan {
         if (d_partial[0]) (void)hipFree(d_partial[0]);
         if (d_partial[1]) (void)hipFree(d_partial[1]);
         if (d_scalars) (void)hipFree(d_scalars);
+        if (d_ticket) (void)hipFree(d_ticket);
         if (h_valid) (void)hipHostFree(h_valid);
     }
 };
@@ -301,6 +303,48 @@ __global__ void __launch_bounds__(kLanes) lbfgs_reduce_kernel(const double *__re
     if (gridDim.x == 1 && e.op != kOpNone) run_epilogue(e, total);
 }
 
+// The last two tree levels in one launch (2 .. 1024 workgroups): every workgroup reduces its
+// group to dst[b], publishes it and takes a ticket; the workgroup that draws the last ticket
+// reduces dst[0 .. gridDim.x) with the same node and runs the scalar epilogue.  The order of
+// the additions is that of two separate launches; only a 5 us launch is saved per dot product.
+// A ticket counter shared by at most 1024 workgroups is cheap; one shared by every workgroup
+// of a streaming pass is not (same-address atomics serialise), which is why level 0 is not
+// folded in as well.
+__global__ void __launch_bounds__(kLanes) lbfgs_reduce_last_two_kernel(const double *__restrict__ src,
+                                                                      uint64_t count, double *dst,
+                                                                      unsigned int *ticket, Epilogue e)
+{
+    __shared__ bool is_last;
+    const uint64_t base = (uint64_t)blockIdx.x * kSlice;
+    const uint64_t left = count - base;
+    double acc = 0.0;
+#pragma unroll
+    for (int u = 0; u < kPerLane; u++) {
+        const uint32_t i = threadIdx.x + u * kLanes;
+        if (i < left) acc = acc + src[base + i];
+    }
+    const double mine = workgroup_tree(acc);
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&dst[blockIdx.x], mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // release dst[b] to the device, acquire what the earlier ticket holders released
+        const unsigned int drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = drawn == gridDim.x - 1;
+    }
+    __syncthreads();      // also separates the two uses of workgroup_tree's shared words
+    if (!is_last) return;
+    double acc2 = 0.0;
+#pragma unroll
+    for (int u = 0; u < kPerLane; u++) {
+        const uint32_t i = threadIdx.x + u * kLanes;
+        if (i < gridDim.x) acc2 = acc2 + __hip_atomic_load(&dst[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const double total = workgroup_tree(acc2);
+    if (threadIdx.x != 0) return;
+    __hip_atomic_store(&dst[0], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     // ready for the next launch
+    if (e.op != kOpNone) run_epilogue(e, total);
+}
+
 // A list with zero or one slice has no tree level to run: the epilogue takes the value as is.
 __global__ void lbfgs_epilogue_kernel(const double *src, uint64_t count, Epilogue e)
 {
@@ -382,7 +426,9 @@ bool ensure_geometry(Context *ctx, Plan &p, const int *sizes, int n)
     return hip_ok(hipMalloc(&p.d_partial[0], level0 * sizeof(double)), "hipMalloc(lbfgs partial sums)") &&
            hip_ok(hipMalloc(&p.d_partial[1], level1 * sizeof(double)), "hipMalloc(lbfgs partial sums)") &&
            hip_ok(hipMalloc(&p.d_scalars, sizeof(LbScalars)), "hipMalloc(lbfgs scalars)") &&
-           hip_ok(hipMemsetAsync(p.d_scalars, 0, sizeof(LbScalars), ctx->stream), "clear lbfgs scalars");
+           hip_ok(hipMemsetAsync(p.d_scalars, 0, sizeof(LbScalars), ctx->stream), "clear lbfgs scalars") &&
+           hip_ok(hipMalloc(&p.d_ticket, sizeof(unsigned int)), "hipMalloc(lbfgs ticket)") &&
+           hip_ok(hipMemsetAsync(p.d_ticket, 0, sizeof(unsigned int), ctx->stream), "clear lbfgs ticket");
 }
 
 Plan *find_plan(Context *ctx, const int *sizes, int n)
@@ -510,6 +556,11 @@ void launch_reduction(Context *ctx, const Plan &p, const Epilogue &e)
     const Epilogue none{kOpNone, nullptr, nullptr, nullptr, nullptr};
     while (count > 1) {
         const uint64_t next = (count + kSlice - 1) / kSlice;
+        if (next > 1 && next <= (uint64_t)kSlice) {
+            lbfgs_reduce_last_two_kernel<<<(uint32_t)next, kLanes, 0, ctx->stream>>>(
+                p.d_partial[src], count, p.d_partial[src ^ 1], p.d_ticket, e);
+            return;
+        }
         lbfgs_reduce_kernel<<<(uint32_t)next, kLanes, 0, ctx->stream>>>(p.d_partial[src], count,
                                                                         p.d_partial[src ^ 1],
                                                                         next == 1 ? e : none);

@@ -342,3 +342,27 @@ def test_c5_size_dot_and_plain_step(dev):
                 dev.free(h)
         dev.free(rho)
         dev.free(alpha)
+
+
+def test_dot_with_three_tree_levels(dev):
+    # more than 1024 * 1024 slices (1.2e9 elements): a plain level, then the fused last two
+    sizes = [450_000_000, 450_000_000, 300_000_000]
+    lib, D = dev.lib, dev.handle
+    ha = [dev.alloc(4 * k) for k in sizes]
+    hb = [dev.alloc(4 * k) for k in sizes]
+    try:
+        for i, k in enumerate(sizes):
+            assert lib.gm_fill_normal_f32(D, ha[i], k, 900 + i, 0.0, 1.0) == 0
+            assert lib.gm_fill_normal_f32(D, hb[i], k, 950 + i, 0.5, 1.0) == 0
+        out = ctypes.c_float()
+        print("dot product over 1.2e9 elements", flush=True)
+        assert lib.gm_lbfgs_dot(D, pkg.handle_array(ha), pkg.handle_array(hb), 3, pkg.int_array([4 * k for k in sizes]),
+                                ctypes.byref(out)) == 0
+        a = [dev.to_numpy(h, k) for h, k in zip(ha, sizes)]
+        b = [dev.to_numpy(h, k) for h, k in zip(hb, sizes)]
+        print("oracle dot product", flush=True)
+        want = oracle().lbfgs_dot(a, b, TREE)
+        assert F(out.value).view(np.uint32) == want.view(np.uint32), (out.value, want)
+    finally:
+        for h in ha + hb:
+            dev.free(h)
