@@ -170,3 +170,41 @@ def test_special_values(dev, rule, hyper):
             assert np.array_equal(a[ok].view(np.uint32), b[ok].view(np.uint32)), (rule, key)
     finally:
         gpu.close()
+
+
+def random_case(rng):
+    """A random rule, hyper-parameter set and tensor list (sizes from 0 to ~200k, log-uniform)."""
+    rule = ["sgd", "adam", "rmsprop", "adagrad", "adadelta", "nadam"][int(rng.integers(0, 6))]
+    f = lambda lo, hi: float(np.float32(10.0 ** rng.uniform(np.log10(lo), np.log10(hi))))
+    wd = 0.0 if rng.random() < 0.4 else f(1e-6, 1e-1)
+    if rule == "sgd":
+        hyper = dict(lr=f(1e-4, 1.0), momentum=0.0 if rng.random() < 0.3 else float(np.float32(rng.uniform(0.1, 0.99))),
+                     weight_decay=wd, nesterov=bool(rng.random() < 0.5))
+    elif rule in ("adam", "nadam"):
+        hyper = dict(lr=f(1e-5, 1e-1), beta1=float(np.float32(rng.uniform(0.5, 0.99))),
+                     beta2=float(np.float32(rng.uniform(0.9, 0.9999))), eps=f(1e-10, 1e-4), weight_decay=wd)
+    elif rule == "rmsprop":
+        hyper = dict(lr=f(1e-4, 1e-1), alpha=float(np.float32(rng.uniform(0.8, 0.999))), eps=f(1e-10, 1e-4),
+                     weight_decay=wd, momentum=0.0 if rng.random() < 0.5 else float(np.float32(rng.uniform(0.1, 0.95))),
+                     centered=bool(rng.random() < 0.5))
+    elif rule == "adagrad":
+        hyper = dict(lr=f(1e-4, 1.0), eps=f(1e-12, 1e-6), weight_decay=wd)
+    else:
+        hyper = dict(rho=float(np.float32(rng.uniform(0.5, 0.99))), eps=f(1e-8, 1e-4), weight_decay=wd)
+    count = int(rng.integers(1, 13))
+    sizes = [0 if rng.random() < 0.05 else int(2.0 ** rng.uniform(0, 17.6)) for _ in range(count)]
+    return rule, hyper, sizes
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_rules_hyperparameters_and_lists(dev, seed):
+    """Randomised parity: rule, hyper-parameters, list shape, weight and gradient magnitudes all
+    drawn from a seeded generator; 4 steps, every buffer compared bit for bit after each."""
+    rng = np.random.default_rng(1000 + seed)
+    rule, hyper, sizes = random_case(rng)
+    wscale, gscale = 10.0 ** rng.uniform(-3, 1), 10.0 ** rng.uniform(-6, 1)
+    w = [rng.normal(0, wscale, n).astype(np.float32) for n in sizes]
+    print(f"seed {seed}: {rule} {hyper} sizes {sizes}", flush=True)
+    with np.errstate(all="ignore"):
+        run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, gscale, n).astype(np.float32) for n in sizes],
+                 steps=4, check_every=1, nthreads=1)
