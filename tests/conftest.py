@@ -11,3 +11,13 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+def pytest_sessionstart(session):
+    """Loads what is built; builds only when nothing is (a fresh checkout): the library and the
+    CPU checker are git-ignored artefacts."""
+    lib = os.path.join(ROOT, "go-metal_amd", "libgometal_hip.so")
+    oracle_lib = os.path.join(ROOT, "oracle", "liboracle.so")
+    if not os.path.exists(lib) or not os.path.exists(oracle_lib):
+        import __graft_entry__
+        __graft_entry__.build()
