@@ -276,9 +276,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
     ap.add_argument("--history", type=int, default=0, help="L-BFGS workloads: history size (default 10)")
+    ap.add_argument("--rule", default="", choices=["", "sgd", "adam", "rmsprop", "adagrad", "adadelta", "nadam"],
+                    help="run another update rule (with BASELINE's hyper-parameters for it) over the workload's list")
     # launch-shape overrides (gm_set_tuning) for comparing lane widths and chunk sizes; 0 / -1 = default
     ap.add_argument("--chunk", type=int, default=0, help="elements per chunk")
-    ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4")
+    ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4 (0: chosen per launch)")
     ap.add_argument("--nontemporal", type=int, default=-1, help="1 / 0: non-temporal hint on / off")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -299,6 +301,10 @@ def main():
         return bench_lbfgs(args, pkg, dev)
 
     desc, sizes_fn, rule, hyper, grad_std = WORKLOADS[args.workload]
+    if args.rule and args.rule != rule:
+        rule = args.rule
+        hyper = next(h for (_, _, r, h, _) in WORKLOADS.values() if r == rule)
+        desc += f" [rule overridden: {rule}]"
     sizes = sizes_fn()
     n = len(sizes)
     params = sum(sizes)
@@ -366,7 +372,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": desc, "tensors": n, "params": params, "rule": rule, "hyper": hyper,
-                   "launch": {"chunk": args.chunk or "auto", "vec": args.vec or 1,
+                   "launch": {"chunk": args.chunk or "auto", "vec": args.vec or "auto",
                               "nontemporal": args.nontemporal != 0}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,

@@ -8,15 +8,16 @@
 // (b div slices_per_chunk), one VEC-wide group per lane: load every stream
 // once, apply the rule in registers, store every state once, exit.
 //
-// VEC = 1 (one fp32 per lane, global_load_dword) is the default: measured on
-// MI355X it sustains about 85 % of peak HBM bandwidth on the 4-read / 3-write
-// Adam stream, against about 80 % for 8-byte and 72-77 % for 16-byte lanes
-// (global_load_dwordx4), whatever the unrolling or workgroup size.  Short
-// single-pass waves keep reads and writes finely interleaved at the memory
-// controllers; wide, unrolled lanes issue them in bursts.  The wider
-// variants stay selectable (gm_set_tuning) so the comparison can be rerun.
-// The path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS
-// staging, no MFMA.
+// Lane width (VEC fp32 elements per lane) is chosen per launch.  One element per lane
+// (global_load_dword) is the choice for the seven-stream rules on large lists: measured on
+// MI355X it sustains about 82 % of peak HBM bandwidth on the 4-read / 3-write Adam stream over
+// 1B parameters, against about 77 % for 8-byte and 71 % for 16-byte lanes (global_load_dwordx4),
+// whatever the unrolling or workgroup size.  Two elements per lane win for the five-stream rules
+// (SGD-momentum, AdaGrad, plain RMSProp: 78-82 % against 70-77 %) and, narrowly, for every rule
+// on lists under about 64M elements.  Short single-pass waves keep reads and writes finely
+// interleaved at the memory controllers; wide, unrolled lanes issue them in bursts.  Every
+// width stays selectable (gm_set_tuning) so the comparison can be rerun.
+// The path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS staging, no MFMA.
 #include "gm_context.hpp"
 #include "gm_plan.hpp"
 #include "gm_rules.hpp"
@@ -34,13 +35,24 @@ typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 constexpr int kBlock = 256;
 constexpr int kAutoChunkCandidates[] = {65536, 16384, 4096};   // largest first
 constexpr double kAutoChunkMaxIdleFraction = 0.05;
-constexpr int kDefaultVec = 1;
+// fp32 elements per lane when the caller has not fixed it (gm_set_tuning): measured on MI355X, a
+// wave does best with about 2 KB of traffic.  Rules with up to five streams (SGD, AdaGrad, plain
+// RMSProp: 3 reads + 2 writes) gain 3 to 9 points from 8-byte lanes at every list size; the
+// seven-stream rules (Adam, NAdam, AdaDelta) gain 1 to 3 points from them on a 25M list, lose 1 on
+// a 125M list and lose 5 on the 1B list.
+constexpr int kAutoVecStreamLimit = 5;
+constexpr uint64_t kAutoVecSmallList = 1ull << 26;      // elements
+
+static int auto_vec(int streams, uint64_t total_elements)
+{
+    return (streams <= kAutoVecStreamLimit || total_elements < kAutoVecSmallList) ? 2 : 1;
+}
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 constexpr size_t kMaxCachedPlans = 16;
 
 static std::atomic<int> g_chunk_elements{0};   // 0: chosen per plan
 static std::atomic<int> g_nontemporal{1};
-static std::atomic<int> g_vec{kDefaultVec};
+static std::atomic<int> g_vec{0};               // 0: chosen per launch by auto_vec
 
 int current_chunk_elements() { return g_chunk_elements.load(); }
 bool current_nontemporal() { return g_nontemporal.load() != 0; }
@@ -542,7 +554,8 @@ template <class Rule>
 static int launch_rule(const Launch &l, const StepParams &prm, int hip_error_code)
 {
     if (l.plan->num_chunks == 0) return 0;
-    const int vec = current_vec();
+    int vec = current_vec();
+    if (vec == 0) vec = auto_vec(3 + 2 * Rule::NSTATE, l.plan->total_elements);   // w, g, states read; w, states written
     uint32_t grid, shift;
     if (!launch_geometry(*l.plan, vec, grid, shift)) return hip_error_code;
     if (vec == 4) launch_rule_vec<Rule, 4>(l, prm, grid, shift);
@@ -621,16 +634,16 @@ float gm_nadam_mu_next(float beta1, int step_count)
 
 int gm_set_tuning(int chunk_elements, int nontemporal, int vec)
 {
-    const int v = vec == 0 ? kDefaultVec : vec;
+    const int v = vec == 0 ? 4 : vec;        // an automatic width may be 1 or 2: the chunk must suit both
     const int c = chunk_elements;
-    if (v != 1 && v != 2 && v != 4) return -1;
+    if (vec != 0 && v != 1 && v != 2 && v != 4) return -1;
     if (c != 0) {
         // a chunk is a power-of-two number of 256 * vec element slices
         if (c < kBlock * v || c % (kBlock * v) != 0) return -1;
         const int slices = c / (kBlock * v);
         if ((slices & (slices - 1)) != 0) return -1;
     }
-    g_vec.store(v);
+    g_vec.store(vec);
     g_chunk_elements.store(c);
     g_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
     return 0;
@@ -660,7 +673,8 @@ int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     p.momentum = momentum;
     p.weight_decay = weight_decay;
     p.nesterov = nesterov;
-    const int vec = current_vec();
+    int vec = current_vec();
+    if (vec == 0) vec = auto_vec(5, l.plan->total_elements);
     const bool nt = current_nontemporal();
     uint32_t grid, shift;
     if (!launch_geometry(*l.plan, vec, grid, shift)) return -10;
@@ -1046,7 +1060,8 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     const uint32_t chunks = l.plan->num_chunks;
     hipStream_t st = l.ctx->stream;
     if (chunks > 0) {
-        const int vec = current_vec();
+        int vec = current_vec();
+        if (vec == 0) vec = auto_vec(8, l.plan->total_elements);
         const bool nt = current_nontemporal();
         uint32_t grid, shift;
         if (!launch_geometry(*l.plan, vec, grid, shift)) return -6;
