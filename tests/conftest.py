@@ -18,6 +18,7 @@ def pytest_sessionstart(session):
     CPU checker are git-ignored artefacts."""
     lib = os.path.join(ROOT, "go-metal_amd", "libgometal_hip.so")
     oracle_lib = os.path.join(ROOT, "oracle", "liboracle.so")
-    if not os.path.exists(lib) or not os.path.exists(oracle_lib):
+    client = os.path.join(ROOT, "tests", "c_client", "abi_client.bin")
+    if not os.path.exists(lib) or not os.path.exists(oracle_lib) or not os.path.exists(client):
         import __graft_entry__
         __graft_entry__.build()
