@@ -54,6 +54,8 @@ ABI = {
                                                u, fp]),
     "gm_lbfgs_dot": (i, [u, up, up, i, ip, fp]),
     "gm_synchronize": (i, [u]),
+    "gm_wait_for_stream": (i, [u, vp]),
+    "gm_signal_stream": (i, [u, vp]),
     "gm_last_error": (ctypes.c_char_p, []),
     "gm_buffer_length": (ctypes.c_size_t, [u]),
     "gm_bias_corrections": (None, [f, f, i, fp, fp]),

@@ -444,6 +444,29 @@ int gm_synchronize(uintptr_t device)
     return 0;
 }
 
+// Cross-stream ordering without a host wait: an event recorded on one stream, waited for by
+// the other.  The event is created per call and destroyed once recorded and enqueued (HIP keeps
+// it alive until the wait has been satisfied).
+static int order_streams(uintptr_t device, void *caller_stream, bool library_waits)
+{
+    if (device == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -3;
+    if (!make_current(ctx)) return -10;
+    hipStream_t theirs = reinterpret_cast<hipStream_t>(caller_stream);
+    hipStream_t first = library_waits ? theirs : ctx->stream;
+    hipStream_t second = library_waits ? ctx->stream : theirs;
+    hipEvent_t ev = nullptr;
+    if (!hip_ok(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreate")) return -10;
+    const bool ok = hip_ok(hipEventRecord(ev, first), "hipEventRecord") &&
+                    hip_ok(hipStreamWaitEvent(second, ev, 0), "hipStreamWaitEvent");
+    (void)hipEventDestroy(ev);
+    return ok ? 0 : -10;
+}
+
+int gm_wait_for_stream(uintptr_t device, void *hip_stream) { return order_streams(device, hip_stream, true); }
+int gm_signal_stream(uintptr_t device, void *hip_stream) { return order_streams(device, hip_stream, false); }
+
 int gm_timer_start(uintptr_t device)
 {
     if (device == 0) return -1;

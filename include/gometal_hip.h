@@ -217,6 +217,15 @@ int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffe
  * -1: device 0; -3: no GPU; -10: HIP error (a kernel fault surfaces here). */
 int gm_synchronize(uintptr_t device);
 
+/* Ordering against a caller's own HIP stream without a host wait (hip_stream is a hipStream_t;
+ * NULL is the legacy default stream).  gm_wait_for_stream: work the library enqueues after the
+ * call starts only when everything enqueued on hip_stream before the call has finished (use it
+ * after producing gradients on that stream).  gm_signal_stream: work enqueued on hip_stream after
+ * the call starts only when everything the library has enqueued so far has finished (use it
+ * before consuming updated weights on that stream).  Codes as gm_synchronize. */
+int gm_wait_for_stream(uintptr_t device, void *hip_stream);
+int gm_signal_stream(uintptr_t device, void *hip_stream);
+
 /* Message of the most recent failure on the calling thread ("" if none). */
 const char *gm_last_error(void);
 

@@ -185,3 +185,50 @@ def test_two_threads_step_two_optimizers(dev):
             oracles[t].step(g)
         compare_snapshots(runs[t].snapshot(), oracles[t].snapshot(), 0, f"thread {t}")
         runs[t].close()
+
+
+def test_ordering_against_a_callers_stream(dev):
+    """Gradients produced on the caller's own HIP stream, the step on the library's stream, the
+    result consumed on the caller's stream again: ordered by gm_wait_for_stream / gm_signal_stream
+    alone, no host wait in between."""
+    hip = ctypes.CDLL("/opt/rocm/lib/libamdhip64.so")
+    hip.hipStreamCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+    hip.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
+    hip.hipHostMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t, ctypes.c_uint]
+    hip.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+    hip.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+    hip.hipHostFree.argtypes = [ctypes.c_void_p]
+    stream = ctypes.c_void_p()
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(stream), 1) == 0          # hipStreamNonBlocking
+    n = 8_000_000
+    nbytes = 4 * n
+    pin_g, pin_out = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipHostMalloc(ctypes.byref(pin_g), nbytes, 0) == 0
+    assert hip.hipHostMalloc(ctypes.byref(pin_out), nbytes, 0) == 0
+    g = np.ctypeslib.as_array(ctypes.cast(pin_g, ctypes.POINTER(ctypes.c_float)), shape=(n,))
+    out = np.ctypeslib.as_array(ctypes.cast(pin_out, ctypes.POINTER(ctypes.c_float)), shape=(n,))
+    rng = np.random.default_rng(21)
+    w0 = rng.normal(0, 0.02, n).astype(np.float32)
+    w, gbuf = dev.from_numpy(w0), dev.alloc(nbytes)
+    lib, D = dev.lib, dev.handle
+    bs = pkg.int_array([nbytes])
+    want = w0.copy()
+    try:
+        for step in range(3):
+            g[:] = rng.normal(0, 1e-2, n).astype(np.float32)
+            want = want - np.float32(0.1) * g
+            assert hip.hipMemcpyAsync(gbuf, pin_g, nbytes, 1, stream) == 0       # H2D on the caller's stream
+            assert lib.gm_wait_for_stream(D, stream) == 0
+            assert lib.execute_sgd_step_mpsgraph(D, arr([w]), arr([gbuf]), None, 1, bs, 0.1, 0.0, 0.0, 0, step + 1) == 0
+            assert lib.gm_signal_stream(D, stream) == 0
+            assert hip.hipMemcpyAsync(pin_out, w, nbytes, 2, stream) == 0        # D2H on the caller's stream
+            assert hip.hipStreamSynchronize(stream) == 0                         # the pinned gradient is reused next
+            assert np.array_equal(out.view(np.uint32), want.view(np.uint32)), step
+        assert lib.gm_wait_for_stream(0, stream) == -1
+    finally:
+        dev.synchronize()
+        hip.hipStreamDestroy(stream)
+        hip.hipHostFree(pin_g)
+        hip.hipHostFree(pin_out)
+        dev.free(w)
+        dev.free(gbuf)
