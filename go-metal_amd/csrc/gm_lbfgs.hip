@@ -48,6 +48,7 @@ constexpr int kPerLane = 4;
 constexpr int kSlice = kLanes * kPerLane;            // 1024: the tree's radix and the slice length
 constexpr int kChunkCandidates[] = {65536, 16384, 4096, 1024};
 constexpr double kMaxIdleFraction = 0.05;
+constexpr int kFusedReduceMaxGroups = 128;
 
 struct alignas(16) LbChunk {
     uint32_t tensor;        // index into the handle rows
@@ -169,7 +170,7 @@ struct StreamArgs {
     const LbChunk *chunks;
     uint32_t slice_shift;
     // rows of the handle table (one device address per tensor); meaning depends on the mode
-    const uintptr_t *r0, *r1, *r2, *r3, *r4;
+    const uintptr_t *r0, *r1, *r2, *r3, *r4, *r5, *r6;
     double *partial;               // slice sums (modes with a dot product)
     const LbScalars *scalars;      // coefficient for kModeAxpy
     float step;                    // kModeUpdate*
@@ -181,6 +182,9 @@ struct StreamArgs {
 //   kModeAxpy            r0 = direction, r1 = v, r2 = dot operand        x = x -/+ c v
 //   kModeUpdate          r0 = direction, r1 = w, r2 = g, r3 = old_g, r4 = s_cur
 //   kModeUpdateFromGrad  same, with r = -g formed in registers (no valid pair this step)
+//                        with DOT, both update modes also run the curvature pass on the values
+//                        they hold: r5 = s_prev, r6 = y_prev; y = g - g', g' being the gradient
+//                        just stored as old_g, and dot(s_prev, y)
 //   kModeCurvature       r0 = g, r1 = old_g, r2 = s_prev, r3 = y_prev    y = g - old_g, dot(s, y)
 //   kModeDotOnly         r0 = a, r1 = b
 template <int MODE, bool DOT, bool NT>
@@ -203,6 +207,12 @@ __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
         p3 = reinterpret_cast<float *>(a.r3[ch.tensor]) + first;
     if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad)
         p4 = reinterpret_cast<float *>(a.r4[ch.tensor]) + first;
+    constexpr bool kFusedCurvature = DOT && (MODE == kModeUpdate || MODE == kModeUpdateFromGrad);
+    float *p5 = nullptr, *p6 = nullptr;
+    if (kFusedCurvature) {
+        p5 = reinterpret_cast<float *>(a.r5[ch.tensor]) + first;
+        p6 = reinterpret_cast<float *>(a.r6[ch.tensor]) + first;
+    }
 
     float coef = 0.0f;
     if (MODE == kModeAxpy) coef = a.scalars->coef;
@@ -218,13 +228,14 @@ __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
     constexpr bool kLoad1 = MODE != kModeInit;
     constexpr bool kLoad2 = kFusedDot || MODE == kModeUpdate || MODE == kModeUpdateFromGrad ||
                             MODE == kModeCurvature;
-    float v0[kPerLane], v1[kPerLane], v2[kPerLane];
+    float v0[kPerLane], v1[kPerLane], v2[kPerLane], v3[kPerLane];
     auto load_element = [&](int u) {
         const size_t o = (size_t)u * kLanes;
         const bool ok = threadIdx.x + u * kLanes < left;
         v0[u] = (kLoad0 && ok) ? ld<NT>(p0 + o) : 0.0f;
         v1[u] = (kLoad1 && ok) ? ld<NT>(p1 + o) : 0.0f;
         v2[u] = (kLoad2 && ok) ? ld<NT>(p2 + o) : 0.0f;
+        v3[u] = (kFusedCurvature && ok) ? ld<NT>(p5 + o) : 0.0f;
     };
     // arithmetic, stores, and the lane's running fp64 sum in element order
     double acc = 0.0;
@@ -252,6 +263,11 @@ __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
             st<NT>(v1[u] + sp, p1 + o);
             st<NT>(g, p3 + o);
             st<NT>(sp, p4 + o);
+            if (kFusedCurvature) {
+                x = g - g;          // y = g - old_g with old_g = g as just stored: +0, or NaN for a non-finite g
+                d = v3[u];
+                st<NT>(x, p6 + o);
+            }
         } else if (MODE == kModeCurvature) {
             x = v0[u] - v1[u];
             d = v2[u];
@@ -303,13 +319,13 @@ __global__ void __launch_bounds__(kLanes) lbfgs_reduce_kernel(const double *__re
     if (gridDim.x == 1 && e.op != kOpNone) run_epilogue(e, total);
 }
 
-// The last two tree levels in one launch (2 .. 1024 workgroups): every workgroup reduces its
+// The last two tree levels in one launch (2 .. kFusedReduceMaxGroups workgroups): every workgroup reduces its
 // group to dst[b], publishes it and takes a ticket; the workgroup that draws the last ticket
 // reduces dst[0 .. gridDim.x) with the same node and runs the scalar epilogue.  The order of
 // the additions is that of two separate launches; only a 5 us launch is saved per dot product.
-// A ticket counter shared by at most 1024 workgroups is cheap; one shared by every workgroup
-// of a streaming pass is not (same-address atomics serialise), which is why level 0 is not
-// folded in as well.
+// Each workgroup's release makes its result visible device-wide, which costs a cache write-back:
+// with 24 workgroups (25M parameters) the launch takes 5 us against 9 for two launches, with 966
+// (1B parameters) it took 24 us, so lists with more groups use two plain launches.
 __global__ void __launch_bounds__(kLanes) lbfgs_reduce_last_two_kernel(const double *__restrict__ src,
                                                                       uint64_t count, double *dst,
                                                                       unsigned int *ticket, Epilogue e)
@@ -556,7 +572,7 @@ void launch_reduction(Context *ctx, const Plan &p, const Epilogue &e)
     const Epilogue none{kOpNone, nullptr, nullptr, nullptr, nullptr};
     while (count > 1) {
         const uint64_t next = (count + kSlice - 1) / kSlice;
-        if (next > 1 && next <= (uint64_t)kSlice) {
+        if (next > 1 && next <= (uint64_t)kFusedReduceMaxGroups) {
             lbfgs_reduce_last_two_kernel<<<(uint32_t)next, kLanes, 0, ctx->stream>>>(
                 p.d_partial[src], count, p.d_partial[src ^ 1], p.d_ticket, e);
             return;
@@ -657,11 +673,23 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uin
     base.scalars = p.d_scalars;
     base.step = initial_step;
 
+    // The curvature pass (y_prev = g - old_g, s_prev . y_prev) reads old_g right after the update
+    // pass has stored g into it, so it can ride on the update pass with the values in registers,
+    // unless the ring has one slot (s_prev is then the s the update pass is writing).
+    const int prev = (history_index - 1 + m) % m;
+    const bool fuse_curvature = history_count > 0 && prev != history_index;
+    auto with_curvature = [&](StreamArgs a) {
+        a.r5 = r.s(prev, n);
+        a.r6 = r.y(prev, n);
+        return a;
+    };
+
     if (valid.empty()) {
         // q = -g, no recursion, p = -q: one pass
         StreamArgs a = base;
         a.r0 = r.dir; a.r1 = r.w; a.r2 = r.g; a.r3 = r.old_g; a.r4 = r.s(history_index, n);
-        launch_stream<kModeUpdateFromGrad, false>(ctx, p, a);
+        if (fuse_curvature) launch_stream<kModeUpdateFromGrad, true>(ctx, p, with_curvature(a));
+        else launch_stream<kModeUpdateFromGrad, false>(ctx, p, a);
     } else {
         const int count = (int)valid.size();
         // q = -g, with the first dot product of the backward loop
@@ -696,16 +724,18 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uin
         // p = -r; x += a p; old_g = g; s_cur = a p  (:1219-1276)
         StreamArgs a = base;
         a.r0 = r.dir; a.r1 = r.w; a.r2 = r.g; a.r3 = r.old_g; a.r4 = r.s(history_index, n);
-        launch_stream<kModeUpdate, false>(ctx, p, a);
+        if (fuse_curvature) launch_stream<kModeUpdate, true>(ctx, p, with_curvature(a));
+        else launch_stream<kModeUpdate, false>(ctx, p, a);
     }
     if (step_size) *step_size = initial_step;
 
     // y_prev = g - old_g, rho_prev = 1 / (s_prev . y_prev)  (:1279-1335)
     if (history_count > 0) {
-        const int prev = (history_index - 1 + m) % m;
-        StreamArgs a = base;
-        a.r0 = r.g; a.r1 = r.old_g; a.r2 = r.s(prev, n); a.r3 = r.y(prev, n);
-        launch_stream<kModeCurvature, true>(ctx, p, a);
+        if (!fuse_curvature) {
+            StreamArgs a = base;
+            a.r0 = r.g; a.r1 = r.old_g; a.r2 = r.s(prev, n); a.r3 = r.y(prev, n);
+            launch_stream<kModeCurvature, true>(ctx, p, a);
+        }
         launch_reduction(ctx, p, Epilogue{kOpRho, nullptr, nullptr, rho_ptr(prev), p.d_scalars});
     }
     return hip_ok(hipGetLastError(), "L-BFGS kernel launch") ? 0 : -8;
