@@ -115,3 +115,19 @@ def test_lbfgs_nil_device_and_history_checks_need_no_gpu():
     assert lib.execute_lbfgs_step_mpsgraph(0, *args, ctypes.byref(step)) == -1      # bridge_optimizer.m:1005-1009
     assert lib.execute_lbfgs_step_mpsgraph_pooled(0, *args, 0x2000, ctypes.byref(step)) == -1
     assert step.value == -1.0
+
+
+def test_prototypes_equal_the_references_cgo_preamble():
+    """Return and parameter types of every function the reference's cgo preamble also declares
+    (tests/golden/reference_prototypes.json, extracted from cgo_bridge/bridge.go) are the same in
+    include/gometal_hip.h: the Go wrappers would compile against this header unchanged."""
+    import json
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
+    import make_reference_prototypes as gen
+    with open(os.path.join(ROOT, "tests", "golden", "reference_prototypes.json")) as f:
+        ref = json.load(f)["prototypes"]
+    mine = gen.header_prototypes()
+    assert len(ref) == 26
+    for name, proto in ref.items():
+        assert mine[name] == proto, (name, mine[name], proto)
