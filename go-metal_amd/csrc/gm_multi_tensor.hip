@@ -363,17 +363,20 @@ multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, 
 // ---- mixed precision ----
 
 // Loss-scale state machine, resident in HBM next to the tensors.
-struct AmpDeviceState {
+struct alignas(16) AmpDeviceState {
+    // head: the 16 bytes every workgroup of the update kernel reads with one scalar load
     float scale;
-    int growth_tracker;
+    float inv_scale;        // 1.0f / scale, kept by whoever changes scale (IEEE division on host and device alike)
     int found_inf;          // set by the check kernel, consumed and cleared by the epilogue
     int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
+    // tail
+    int growth_tracker;
     int last_skipped;
     float growth_factor;
     float backoff_factor;
     int growth_interval;
     int skipped_steps;      // steps dropped so far
-    int pad;
+    int pad[2];
 };
 
 // Bias corrections for the asynchronous step.  The host does not know how many of the steps
@@ -441,13 +444,31 @@ __global__ void __launch_bounds__(kBlock)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
                        const AmpDeviceState *__restrict__ state, AmpBiasTable bias)
 {
-    if (state->found_inf) return;
-    const float inv_scale = 1.0f / state->scale;
-    int pick = bias.count > 1 ? state->applied_steps - bias.base : 0;
-    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
-    prm.bc1 = bias.bc1[pick];
-    prm.bc2 = bias.bc2[pick];
+    // The state's head (scale, its reciprocal, flag, applied steps) comes with one 16-byte scalar load
+    // and the chunk descriptor with another, both issued before anything is decided; the bias
+    // table sits in the kernel arguments and its entry is picked by scalar selects.  No load
+    // waits for another except on the kernel-argument pointers themselves.
+    const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * kBlock * VEC;
+    // (the weight pointer is never null; testing it here makes the compiler fetch the whole
+    // descriptor before the branch instead of the count first and the addresses after it)
+    if ((head.z != 0u) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
+        return;                                                        // step dropped, or an idle slice
+    const float inv_scale = __uint_as_float(head.y);
+    const int applied = (int)head.w;
+    int pick = bias.count > 1 ? applied - bias.base : 0;
+    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
+    float bc1 = bias.bc1[0], bc2 = bias.bc2[0];
+#pragma unroll
+    for (int j = 1; j < kAmpMaxInFlight; j++) {
+        if (pick == j) {
+            bc1 = bias.bc1[j];
+            bc2 = bias.bc2[j];
+        }
+    }
+    prm.bc1 = bc1;
+    prm.bc2 = bc2;
     update_slice<AdamRule, VEC, NT, true>(ch, slice_shift, prm, inv_scale);
 }
 
@@ -472,6 +493,7 @@ __global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_
             st.growth_tracker = 0;
         }
     }
+    st.inv_scale = 1.0f / st.scale;
     st.last_skipped = found ? 1 : 0;
     st.found_inf = 0;
     *state = st;
@@ -934,6 +956,7 @@ uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_f
     if (ok) {
         std::memset(s->h_pinned, 0, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState));
         s->h_pinned->scale = init_scale;
+        s->h_pinned->inv_scale = 1.0f / init_scale;
         s->h_pinned->growth_factor = growth_factor;
         s->h_pinned->backoff_factor = backoff_factor;
         s->h_pinned->growth_interval = growth_interval;
@@ -990,6 +1013,7 @@ int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
     std::lock_guard<std::mutex> lk(s->ctx->mu);
     if (!amp_download(s)) return -6;
     s->h_pinned->scale = scale;
+    s->h_pinned->inv_scale = 1.0f / scale;
     s->h_pinned->growth_tracker = growth_tracker;
     return amp_upload(s) ? 0 : -6;
 }
