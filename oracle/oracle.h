@@ -114,8 +114,9 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
  *
  * Pinning status: the reference's tests assert no numerical output of this function
  * (optimizer/lbfgs_test.go checks construction, counters and error strings only).  The
- * statement order is pinned by tests/golden/lbfgs_kat.json, written by an independent
- * Python evaluator (numpy float32 element ops; Python floats for the fp64 tree), by the
+ * statement order is pinned by tests/golden/lbfgs_kat.json, written by two independent
+ * evaluators that must agree bit for bit (numpy float32 element ops with Python floats for
+ * the fp64 tree; exact rational arithmetic rounded by integer arithmetic), by the
  * closed form w' = w + initial_step * g for an empty history, and, for GM_ORACLE_DOT_TREE,
  * by agreement with the exactly rounded dot product (math.fsum) to 1 ulp. */
 enum { GM_ORACLE_DOT_REFERENCE = 0, GM_ORACLE_DOT_TREE = 1 };

@@ -2,14 +2,21 @@
 """Writes tests/golden/lbfgs_kat.json: known-answer vectors for the L-BFGS step
 (cgo_bridge/bridge_optimizer.m:980-1321).
 
-The evaluator here shares no code with oracle/oracle_lbfgs.c or the HIP kernels:
-element operations are numpy float32 ufunc calls (one rounding each), the
-reference-order dot product is a Python loop over numpy float32 scalars, and the
-tree-order dot product runs on Python floats (binary64) with the product of two
-binary32 values formed exactly.  The reference asserts no numerical output for
-this function, so the expected values come from this evaluator; what they pin is
-the statement order of the reference's loop nest (see the notes in
-oracle/oracle_lbfgs.c) and the two summation orders.
+Two evaluators, neither sharing code with oracle/oracle_lbfgs.c or the HIP kernels,
+must agree bit for bit on every case before the file is written:
+
+  * numpy: element operations are float32 ufunc calls (one rounding each), the
+    reference-order dot product is a Python loop over numpy float32 scalars, and the
+    tree-order dot product runs on Python floats (binary64) with the product of two
+    binary32 values formed exactly;
+  * exact: every operation is carried out over the rationals (fractions.Fraction)
+    and rounded to binary32 -- or, inside the tree, to binary64 -- by integer
+    arithmetic (make_golden.round_to_format): "what IEEE-754 fixes" for the
+    statement sequence.
+
+The reference asserts no numerical output for this function, so the expected values
+come from these evaluators; what they pin is the statement order of the reference's
+loop nest (see the notes in oracle/oracle_lbfgs.c) and the two summation orders.
 
 Run from the repo root:  python tests/golden/make_lbfgs_golden.py
 """
@@ -17,9 +24,14 @@ import hashlib
 import json
 import os
 
+import sys
+from fractions import Fraction
+
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+from make_golden import f32_bits, rf32, round_to_format  # noqa: E402  (exact rounding helpers)
 F = np.float32
 SLICE, LANES = 1024, 256
 
@@ -106,6 +118,109 @@ def lbfgs_step(st, g, m, count, index, step, mode):
                 st["y"][prev][i] = np.subtract(g[i], st["old_g"][i], dtype=F)
             sdy = dot(st["s"][prev], st["y"][prev], mode, False)
             st["rho"][prev] = F(1.0) / sdy if abs(float(sdy)) > 1e-10 else F(0.0)
+
+
+# ----------------------------------------------------------------------------
+# the exact evaluator (finite values only: the golden cases hold no inf / NaN)
+# ----------------------------------------------------------------------------
+def rf64(x):
+    r = round_to_format(x, 52, -1022, 1023)
+    assert not isinstance(r, str)
+    return r
+
+
+def exact_node(values):
+    lanes = []
+    for l in range(LANES):
+        acc = Fraction(0)
+        for i in range(l, min(len(values), SLICE), LANES):
+            acc = rf64(acc + values[i])
+        lanes.append(acc)
+    while len(lanes) > 1:
+        lanes = [rf64(lanes[i] + lanes[i + 1]) for i in range(0, len(lanes), 2)]
+    return lanes[0]
+
+
+def exact_dot(a, b, mode, per_tensor):
+    if mode == "tree":
+        level = []
+        for ta, tb in zip(a, b):
+            for off in range(0, len(ta), SLICE):
+                level.append(exact_node([x * y for x, y in zip(ta[off:off + SLICE], tb[off:off + SLICE])]))
+        if not level:
+            return Fraction(0)
+        while len(level) > 1:
+            level = [exact_node(level[i:i + SLICE]) for i in range(0, len(level), SLICE)]
+        return rf32(level[0])
+    total = Fraction(0)
+    for ta, tb in zip(a, b):
+        if per_tensor:
+            d = Fraction(0)
+            for x, y in zip(ta, tb):
+                d = rf32(d + rf32(x * y))
+            total = rf32(total + d)
+        else:
+            for x, y in zip(ta, tb):
+                total = rf32(total + rf32(x * y))
+    return total
+
+
+def exact_state(st):
+    fr = lambda t: [Fraction(float(v)) for v in t]
+    return {"w": [fr(t) for t in st["w"]], "old_g": [fr(t) for t in st["old_g"]], "dir": [fr(t) for t in st["dir"]],
+            "s": [[fr(t) for t in h] for h in st["s"]], "y": [[fr(t) for t in h] for h in st["y"]],
+            "rho": fr(st["rho"]), "alpha": fr(st["alpha"])}
+
+
+def exact_step(st, g, m, count, index, step, mode):
+    n = len(g)
+    limit = Fraction(1, 10 ** 10)          # the double constant 1e-10 differs from 10^-10 by 4e-27; no rho comes that close
+    st["dir"] = [[-x for x in t] for t in g]
+    for j in range(count - 1, -1, -1):
+        idx = (index - count + j + m) % m
+        rho = st["rho"][idx]
+        if abs(rho) < limit:
+            st["alpha"][j] = Fraction(0)
+            continue
+        a = rf32(exact_dot(st["s"][idx], st["dir"], mode, True) * rho)
+        st["alpha"][j] = a
+        st["dir"] = [[rf32(x - rf32(a * y)) for x, y in zip(st["dir"][i], st["y"][idx][i])] for i in range(n)]
+    for j in range(count):
+        idx = (index - count + j + m) % m
+        rho = st["rho"][idx]
+        if abs(rho) < limit:
+            continue
+        beta = rf32(exact_dot(st["y"][idx], st["dir"], mode, True) * rho)
+        coeff = rf32(st["alpha"][j] - beta)
+        st["dir"] = [[rf32(x + rf32(coeff * sv)) for x, sv in zip(st["dir"][i], st["s"][idx][i])] for i in range(n)]
+    st["dir"] = [[-x for x in t] for t in st["dir"]]
+    a = Fraction(float(F(step)))
+    st["w"] = [[rf32(w + rf32(a * p)) for w, p in zip(st["w"][i], st["dir"][i])] for i in range(n)]
+    st["old_g"] = [list(t) for t in g]
+    st["s"][index] = [[rf32(a * p) for p in st["dir"][i]] for i in range(n)]
+    if count > 0:
+        prev = (index - 1 + m) % m
+        st["y"][prev] = [[rf32(x - o) for x, o in zip(g[i], st["old_g"][i])] for i in range(n)]
+        sdy = exact_dot(st["s"][prev], st["y"][prev], mode, False)
+        st["rho"][prev] = rf32(Fraction(1) / sdy) if abs(sdy) > limit else Fraction(0)
+
+
+def exact_bits(t):
+    # a zero result carries no sign here; the numpy evaluator's -0.0 (from -g with g = +0) never
+    # occurs in the cases (gradients are non-zero) and x - x gives +0 in both
+    return [f32_bits(v) for v in t]
+
+
+def assert_same_as_exact(cur, ex, where):
+    for key in ("w", "old_g", "dir"):
+        for i, t in enumerate(cur[key]):
+            assert bits(t) == exact_bits(ex[key][i]), (where, key, i)
+    for key in ("s", "y"):
+        for h, tensors in enumerate(cur[key]):
+            for i, t in enumerate(tensors):
+                assert bits(t) == exact_bits(ex[key][h][i]), (where, key, h, i)
+    assert bits(cur["rho"]) == exact_bits(ex["rho"]), (where, "rho")
+    assert bits(cur["alpha"]) == exact_bits(ex["alpha"]), (where, "alpha")
 
 
 def formula_array(seed, n, scale):
@@ -201,10 +316,13 @@ def make_case(name, rng, sizes, m, count, index, steps, step_size, seeded_histor
         case["init_digest"] = digest(st)
     for mode in ("reference", "tree"):
         cur = clone(st)
+        ex = exact_state(st)
         c, hi = count, index
         out = []
-        for g in grads:
+        for k, g in enumerate(grads):
             lbfgs_step(cur, g, m, c, hi, step_size, mode)
+            exact_step(ex, [[Fraction(float(v)) for v in t] for t in g], m, c, hi, step_size, mode)
+            assert_same_as_exact(cur, ex, (name, mode, k))     # the two evaluators must agree exactly
             hi = (hi + 1) % m                      # optimizer/lbfgs.go:287-290
             c = min(c + 1, m)
             if formula_seed is None:
