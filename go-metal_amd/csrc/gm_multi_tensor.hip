@@ -13,8 +13,7 @@
 // MI355X it sustains about 82 % of peak HBM bandwidth on the 4-read / 3-write Adam stream over
 // 1B parameters, against about 77 % for 8-byte and 71 % for 16-byte lanes (global_load_dwordx4),
 // whatever the unrolling or workgroup size.  Two elements per lane win for the five-stream rules
-// (SGD-momentum, AdaGrad, plain RMSProp: 78-82 % against 70-77 %) and, narrowly, for every rule
-// on lists under about 64M elements.  Short single-pass waves keep reads and writes finely
+// (SGD-momentum, AdaGrad, plain RMSProp: 79-80 % against 71-77 %).  Short single-pass waves keep reads and writes finely
 // interleaved at the memory controllers; wide, unrolled lanes issue them in bursts.  Every
 // width stays selectable (gm_set_tuning) so the comparison can be rerun.
 // The path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS staging, no MFMA.
@@ -35,17 +34,16 @@ typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 constexpr int kBlock = 256;
 constexpr int kAutoChunkCandidates[] = {65536, 16384, 4096};   // largest first
 constexpr double kAutoChunkMaxIdleFraction = 0.05;
-// fp32 elements per lane when the caller has not fixed it (gm_set_tuning): measured on MI355X, a
-// wave does best with about 2 KB of traffic.  Rules with up to five streams (SGD, AdaGrad, plain
-// RMSProp: 3 reads + 2 writes) gain 3 to 9 points from 8-byte lanes at every list size; the
-// seven-stream rules (Adam, NAdam, AdaDelta) gain 1 to 3 points from them on a 25M list, lose 1 on
-// a 125M list and lose 5 on the 1B list.
+// fp32 elements per lane when the caller has not fixed it (gm_set_tuning), measured on MI355X over
+// lists of 25M, 125M and 1B parameters: rules with five streams (SGD-momentum, AdaGrad, plain
+// RMSProp: 3 reads + 2 writes) run at 79-80 % of peak with 8-byte lanes against 71-77 % with
+// 4-byte lanes at every size; the seven-stream rules (Adam, NAdam, AdaDelta) run at 81-82 %
+// with 4-byte lanes against 76-79 % on the larger lists and within a point either way on 25M.
 constexpr int kAutoVecStreamLimit = 5;
-constexpr uint64_t kAutoVecSmallList = 1ull << 26;      // elements
 
-static int auto_vec(int streams, uint64_t total_elements)
+static int auto_vec(int streams)
 {
-    return (streams <= kAutoVecStreamLimit || total_elements < kAutoVecSmallList) ? 2 : 1;
+    return streams <= kAutoVecStreamLimit ? 2 : 1;
 }
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 constexpr size_t kMaxCachedPlans = 16;
@@ -577,7 +575,7 @@ static int launch_rule(const Launch &l, const StepParams &prm, int hip_error_cod
 {
     if (l.plan->num_chunks == 0) return 0;
     int vec = current_vec();
-    if (vec == 0) vec = auto_vec(3 + 2 * Rule::NSTATE, l.plan->total_elements);   // w, g, states read; w, states written
+    if (vec == 0) vec = auto_vec(3 + 2 * Rule::NSTATE);   // w, g, states read; w, states written
     uint32_t grid, shift;
     if (!launch_geometry(*l.plan, vec, grid, shift)) return hip_error_code;
     if (vec == 4) launch_rule_vec<Rule, 4>(l, prm, grid, shift);
@@ -696,7 +694,7 @@ int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     p.weight_decay = weight_decay;
     p.nesterov = nesterov;
     int vec = current_vec();
-    if (vec == 0) vec = auto_vec(5, l.plan->total_elements);
+    if (vec == 0) vec = auto_vec(5);
     const bool nt = current_nontemporal();
     uint32_t grid, shift;
     if (!launch_geometry(*l.plan, vec, grid, shift)) return -10;
@@ -1085,7 +1083,7 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     hipStream_t st = l.ctx->stream;
     if (chunks > 0) {
         int vec = current_vec();
-        if (vec == 0) vec = auto_vec(8, l.plan->total_elements);
+        if (vec == 0) vec = auto_vec(8);
         const bool nt = current_nontemporal();
         uint32_t grid, shift;
         if (!launch_geometry(*l.plan, vec, grid, shift)) return -6;

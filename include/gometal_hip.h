@@ -322,7 +322,7 @@ int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, 
  * 256 * vec, of 1024 when vec is automatic; 0 = default: 65536, 16384 or 4096, the largest
  * that keeps idle workgroups under 5 % for the tensor list), non-temporal memory hints
  * on/off (-1 = default on) and fp32 elements per lane (1, 2 or 4; 0 = default: 2 for rules
- * with up to five streams or lists under 2^26 elements, else 1).
+ * with up to five streams, else 1).
  * -1 if the combination is not valid (nothing changes). */
 int gm_set_tuning(int chunk_elements, int nontemporal, int vec);
 
