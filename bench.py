@@ -219,6 +219,96 @@ def bench_lbfgs(args, pkg, dev):
     print(json.dumps(result))
 
 
+def bench_primitives(args, pkg, dev):
+    """Buffer primitives of the boundary on one large buffer each: zero fill, fp32 <-> fp16 conversion,
+    device-to-device copy (HBM-bound, timed with HIP events on the library's stream) and the host copies
+    in both directions (PCIe-bound, wall time; the caller's array is ordinary pageable memory)."""
+    lib, D = dev.lib, dev.handle
+    elems = 1 << 28                                   # 1 GiB of fp32, 512 MiB of fp16
+    f32, f16, f32b = dev.alloc(4 * elems), dev.alloc(2 * elems), dev.alloc(4 * elems)
+    lib.gm_fill_normal_f32(D, f32, elems, 0x51, 0.0, 1.0)
+    dev.synchronize()
+    shape = pkg.int_array([elems])
+    F32, F16 = 0, 2
+
+    def checked(rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed rc={rc}: {lib.gm_last_error().decode()}")
+
+    cases = {
+        "zero_metal_buffer": (lambda: checked(lib.zero_metal_buffer(D, f32b, 4 * elems), "zero"), 4 * elems),
+        "convert_tensor_type f32->f16": (lambda: checked(lib.convert_tensor_type(f32, f16, shape, 1, F32, F16, D),
+                                                         "convert"), 6 * elems),
+        "convert_tensor_type f16->f32": (lambda: checked(lib.convert_tensor_type(f16, f32b, shape, 1, F16, F32, D),
+                                                         "convert"), 6 * elems),
+        "copy_buffer_to_buffer_sync": (lambda: checked(lib.copy_buffer_to_buffer_sync(f32, f32b, 0, 0, 4 * elems),
+                                                       "copy"), 8 * elems),
+        "gm_copy_probe (16-byte copy kernel)": (lambda: checked(lib.gm_copy_probe(D, f32b, f32, 4 * elems), "probe"),
+                                                8 * elems),
+    }
+    table = {}
+    for name, (launch, nbytes) in cases.items():
+        wall_ms, event_ms = time_steps(dev, launch, args.steps, args.warmup)
+        gbs = nbytes / (event_ms * 1e-3) / 1e9
+        table[name] = {"bytes": nbytes, "kernel_ms": event_ms, "ms_per_call": wall_ms, "achieved": gbs,
+                       "frac": gbs / HBM_PEAK_GBS}
+        print(f"{name}: {event_ms:.4f} ms, {gbs:.0f} GB/s", file=sys.stderr, flush=True)
+
+    host_elems = 1 << 26                              # 256 MiB
+    host = np.random.default_rng(3).standard_normal(host_elems, dtype=np.float32)
+    back = np.empty_like(host)
+    fp = ctypes.POINTER(ctypes.c_float)
+    pcie = {}
+    for name, call in (("copy_float32_array_to_metal_buffer",
+                        lambda: lib.copy_float32_array_to_metal_buffer(f32, host.ctypes.data_as(fp), host_elems)),
+                       ("copy_metal_buffer_to_float32_array",
+                        lambda: lib.copy_metal_buffer_to_float32_array(f32, back.ctypes.data_as(fp), host_elems))):
+        checked(call(), name)
+        t0 = time.perf_counter()
+        reps = 5
+        for _ in range(reps):
+            checked(call(), name)
+        dt = (time.perf_counter() - t0) / reps
+        pcie[name] = {"bytes": 4 * host_elems, "ms_per_call": dt * 1e3, "achieved": 4 * host_elems / dt / 1e9,
+                      "unit": "GB/s", "bound": "pcie, pageable host memory"}
+    if not np.array_equal(host, back):
+        raise RuntimeError("host round trip changed the data")
+
+    result = {"metric": "achieved HBM GB/s of the buffer primitives (% of peak)", "unit": "GB/s", "n_gpus": 1,
+              "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None, "dtype": "f32 / f16 / bytes", "data": "synthetic",
+              "config": {"workload": f"buffer primitives on {elems} elements", "elements": elems}}
+    head = table["convert_tensor_type f32->f16"]
+    result["value"] = head["achieved"]
+    result["ms_per_step"] = head["ms_per_call"]
+    result["roofline"] = {"bound": "hbm", "achieved": head["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": head["frac"], "traffic": None, "kernel": "convert_f32_to_f16_kernel",
+                          "kernel_ms": head["kernel_ms"]}
+    result["primitives"] = table
+    result["host_copies"] = pcie
+    if args.no_cpu_baseline:
+        result["cpu_baseline"] = None
+    else:
+        from oracle_lib import oracle
+        o = oracle()
+        threads = min(16, os.cpu_count() or 1)
+        sample = host
+        o.f32_to_f16(sample, nthreads=threads)
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < 10.0:
+            o.f32_to_f16(sample, nthreads=threads)
+            reps += 1
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": 6 * host_elems * reps / dt / 1e9, "unit": "GB/s", "cores": threads,
+                                  "kind": "port",
+                                  "sample": f"fp32->fp16 conversion of {host_elems} elements, {reps} calls in "
+                                            f"{dt:.1f} s, oracle/oracle.c on {threads} threads"}
+    for h in (f32, f16, f32b):
+        dev.free(h)
+    dev.close()
+    print(json.dumps(result))
+
+
 def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
     """The reference's algorithm as it runs it: one CPU thread, running fp32 sums
     (oracle/oracle_lbfgs.c in reference order), on the leading tensors of the workload."""
@@ -253,7 +343,7 @@ def run_all(args):
     """Every configuration as a child process (this process never touches the GPU)."""
     import subprocess
     results = {}
-    for name in sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS):
+    for name in sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives"]:
         cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", str(args.steps),
                "--warmup", str(args.warmup)]
         if args.no_cpu_baseline:
@@ -271,7 +361,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["all"],
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives", "all"],
                     help="'all': every configuration in turn, each in a process of its own; the line printed "
                          "is the headline configuration's with the others under 'configs'")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -283,6 +373,7 @@ def main():
     ap.add_argument("--chunk", type=int, default=0, help="elements per chunk")
     ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4 (0: chosen per launch)")
     ap.add_argument("--nontemporal", type=int, default=-1, help="1 / 0: non-temporal hint on / off")
+    ap.add_argument("--lanes", type=int, default=0, help="lanes per workgroup of the update kernels: 128 or 256")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the optimizer step shards without communication, and this "
@@ -297,9 +388,13 @@ def main():
     lib, D = dev.lib, dev.handle
     if lib.gm_set_tuning(args.chunk, args.nontemporal, args.vec) != 0:
         sys.exit("invalid --chunk / --vec combination (a chunk is a power-of-two multiple of 256 * vec elements)")
+    if lib.gm_set_workgroup_lanes(args.lanes) != 0:
+        sys.exit("invalid --lanes (128 or 256)")
 
     if args.workload in LBFGS_WORKLOADS:
         return bench_lbfgs(args, pkg, dev)
+    if args.workload == "primitives":
+        return bench_primitives(args, pkg, dev)
 
     desc, sizes_fn, rule, hyper, grad_std = WORKLOADS[args.workload]
     if args.rule and args.rule != rule:
@@ -373,7 +468,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": desc, "tensors": n, "params": params, "rule": rule, "hyper": hyper,
-                   "launch": {"chunk": args.chunk or "auto", "vec": args.vec or "auto",
+                   "launch": {"chunk": args.chunk or "auto", "vec": args.vec or "auto", "lanes": args.lanes or "auto",
                               "nontemporal": args.nontemporal != 0}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,

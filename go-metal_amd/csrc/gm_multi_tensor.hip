@@ -2,21 +2,21 @@
 // the execute_*_step entry points of the C ABI (the HIP counterpart of
 // cgo_bridge/bridge_optimizer.m).
 //
-// One launch per step.  The parameter list is cut into chunks of
-// chunk_elements (4096 to 65536, chosen per list) and each chunk into slices of 256 * VEC
-// elements; workgroup b handles slice (b mod slices_per_chunk) of chunk
-// (b div slices_per_chunk), one VEC-wide group per lane: load every stream
-// once, apply the rule in registers, store every state once, exit.
+// One launch per step.  The parameter list is cut into chunks of chunk_elements (4096 to 65536,
+// chosen per list) and each chunk into slices of BLOCK * VEC elements; workgroup b handles slice
+// (b mod slices_per_chunk) of chunk (b div slices_per_chunk), one VEC-wide group per lane: load
+// every stream once, apply the rule in registers, store every state once, exit.
 //
-// Lane width (VEC fp32 elements per lane) is chosen per launch.  One element per lane
-// (global_load_dword) is the choice for the seven-stream rules on large lists: measured on
-// MI355X it sustains about 82 % of peak HBM bandwidth on the 4-read / 3-write Adam stream over
-// 1B parameters, against about 77 % for 8-byte and 71 % for 16-byte lanes (global_load_dwordx4),
-// whatever the unrolling or workgroup size.  Two elements per lane win for the five-stream rules
-// (SGD-momentum, AdaGrad, plain RMSProp: 79-80 % against 71-77 %).  Short single-pass waves keep reads and writes finely
-// interleaved at the memory controllers; wide, unrolled lanes issue them in bursts.  Every
-// width stays selectable (gm_set_tuning) so the comparison can be rerun.
-// The path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS staging, no MFMA.
+// Lane width (VEC fp32 elements per lane) and workgroup size (BLOCK lanes) are chosen per launch
+// by the number of streams the rule touches.  One element per lane (global_load_dword) in
+// 256-lane workgroups is the choice for the seven-stream rules: measured on MI355X it sustains
+// about 82 % of peak HBM bandwidth on the 4-read / 3-write Adam stream over 1B parameters,
+// against about 77 % for 8-byte and 71 % for 16-byte lanes (global_load_dwordx4), whatever the
+// unrolling.  The five-stream rules (SGD-momentum, AdaGrad, plain RMSProp) do best with two
+// elements per lane in 128-lane workgroups (81-83 %).  Short single-pass waves keep reads and
+// writes finely interleaved at the memory controllers; wide, unrolled lanes issue them in bursts.
+// Every shape stays selectable (gm_set_tuning, gm_set_workgroup_lanes) so the comparison can be
+// rerun.  The path is HBM-bound (about 20 flops per 28 bytes for Adam): no LDS staging, no MFMA.
 #include "gm_context.hpp"
 #include "gm_plan.hpp"
 #include "gm_rules.hpp"
@@ -34,33 +34,34 @@ typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 constexpr int kBlock = 256;
 constexpr int kAutoChunkCandidates[] = {65536, 16384, 4096};   // largest first
 constexpr double kAutoChunkMaxIdleFraction = 0.05;
-// fp32 elements per lane when the caller has not fixed it (gm_set_tuning), measured on MI355X over
-// lists of 25M, 125M and 1B parameters: rules with five streams (SGD-momentum, AdaGrad, plain
-// RMSProp: 3 reads + 2 writes) run at 79-80 % of peak with 8-byte lanes against 71-77 % with
-// 4-byte lanes at every size; the seven-stream rules (Adam, NAdam, AdaDelta) run at 81-82 %
-// with 4-byte lanes against 76-79 % on the larger lists and within a point either way on 25M.
-constexpr int kAutoVecStreamLimit = 5;
+// Launch shape when the caller has not fixed it (gm_set_tuning, gm_set_workgroup_lanes), measured on
+// MI355X over lists of 25M, 125M and 1B parameters.  Rules with five streams (SGD-momentum, AdaGrad,
+// plain RMSProp: 3 reads + 2 writes): 8-byte lanes in 128-lane workgroups, 81-83 % of peak, against
+// 76-82 % in 256-lane workgroups and 71-77 % with 4-byte lanes.  Seven streams and more (Adam, NAdam,
+// AdaDelta, the mixed-precision step): 4-byte lanes in 256-lane workgroups, 81-82 %, against 79-80 %
+// in 128-lane workgroups and 76-79 % with 8-byte lanes.
+constexpr int kAutoFewStreams = 5;
 
-static int auto_vec(int streams)
-{
-    return streams <= kAutoVecStreamLimit ? 2 : 1;
-}
+static int auto_vec(int streams) { return streams <= kAutoFewStreams ? 2 : 1; }
+static int auto_block(int streams) { return streams <= kAutoFewStreams ? 128 : kBlock; }
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 constexpr size_t kMaxCachedPlans = 16;
 
 static std::atomic<int> g_chunk_elements{0};   // 0: chosen per plan
 static std::atomic<int> g_nontemporal{1};
 static std::atomic<int> g_vec{0};               // 0: chosen per launch by auto_vec
+static std::atomic<int> g_block{0};             // lanes per workgroup of the update kernels; 0: auto_block
 
 int current_chunk_elements() { return g_chunk_elements.load(); }
 bool current_nontemporal() { return g_nontemporal.load() != 0; }
 int current_vec() { return g_vec.load(); }
+int current_block() { return g_block.load(); }
 
 // log2(slices per chunk) for a chunk size and lane width; chunk_elements is a
 // power-of-two multiple of 256 * vec (gm_set_tuning enforces it).
-static uint32_t slice_shift_for(int chunk_elements, int vec)
+static uint32_t slice_shift_for(int chunk_elements, int vec, int block)
 {
-    uint32_t slices = (uint32_t)(chunk_elements / (kBlock * vec));
+    uint32_t slices = (uint32_t)(chunk_elements / (block * vec));
     uint32_t shift = 0;
     while ((1u << shift) < slices) shift++;
     return shift;
@@ -322,12 +323,12 @@ __device__ inline void update_group(const Chunk &ch, uint32_t first, const StepP
 }
 
 // Workgroup b -> (chunk, slice).  slice_shift = log2(slices per chunk).
-template <class Rule, int VEC, bool NT, bool AMP>
+template <class Rule, int VEC, bool NT, bool AMP, int BLOCK>
 __device__ inline void update_slice(const Chunk &ch, uint32_t slice_shift, const StepParams &prm,
                                     float inv_scale)
 {
     const uint32_t slice = blockIdx.x & ((1u << slice_shift) - 1u);
-    const uint32_t local = (slice * kBlock + threadIdx.x) * VEC;   // first element of this lane within the chunk
+    const uint32_t local = (slice * BLOCK + threadIdx.x) * VEC;   // first element of this lane within the chunk
     if (local >= ch.count) return;
     constexpr uint32_t vec_flag = VEC == 4 ? kRecVec4Ok : kRecVec2Ok;
     if (VEC > 1 && (ch.flags & vec_flag) && local + VEC <= ch.count) {
@@ -338,24 +339,24 @@ __device__ inline void update_slice(const Chunk &ch, uint32_t slice_shift, const
     }
 }
 
-template <class Rule, int VEC, bool NT>
-__global__ void __launch_bounds__(kBlock)
+template <class Rule, int VEC, bool NT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
 multi_tensor_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm)
 {
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
-    update_slice<Rule, VEC, NT, false>(ch, slice_shift, prm, 1.0f);
+    update_slice<Rule, VEC, NT, false, BLOCK>(ch, slice_shift, prm, 1.0f);
 }
 
 // SGD: a tensor without a momentum buffer takes the vanilla rule.
-template <int VEC, bool NT>
-__global__ void __launch_bounds__(kBlock)
+template <int VEC, bool NT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
 multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm)
 {
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
     if (prm.momentum > 0.0f && ch.p[kSlotState0] != nullptr)
-        update_slice<SgdMomentumRule, VEC, NT, false>(ch, slice_shift, prm, 1.0f);
+        update_slice<SgdMomentumRule, VEC, NT, false, BLOCK>(ch, slice_shift, prm, 1.0f);
     else
-        update_slice<SgdVanillaRule, VEC, NT, false>(ch, slice_shift, prm, 1.0f);
+        update_slice<SgdVanillaRule, VEC, NT, false, BLOCK>(ch, slice_shift, prm, 1.0f);
 }
 
 // ---- mixed precision ----
@@ -437,8 +438,8 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__re
 
 // Phase B: the Adam update on unscaled gradients, skipped as a whole when the
 // flag is set.
-template <int VEC, bool NT>
-__global__ void __launch_bounds__(kBlock)
+template <int VEC, bool NT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
                        const AmpDeviceState *__restrict__ state, AmpBiasTable bias)
 {
@@ -448,7 +449,7 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     // waits for another except on the kernel-argument pointers themselves.
     const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
-    const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * kBlock * VEC;
+    const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
     // (the weight pointer is never null; testing it here makes the compiler fetch the whole
     // descriptor before the branch instead of the count first and the addresses after it)
     if ((head.z != 0u) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
@@ -467,7 +468,7 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     }
     prm.bc1 = bc1;
     prm.bc2 = bc2;
-    update_slice<AdamRule, VEC, NT, true>(ch, slice_shift, prm, inv_scale);
+    update_slice<AdamRule, VEC, NT, true, BLOCK>(ch, slice_shift, prm, inv_scale);
 }
 
 // Epilogue (one lane, same stream, after phase B has drained): advances the
@@ -546,9 +547,9 @@ static int prepare(uintptr_t device, const PlanRequest &req, int hip_error_code,
 
 // Grid size: every chunk gets the same number of slices; the slices past the
 // end of a short chunk exit at once.
-static bool launch_geometry(const MultiTensorPlan &plan, int vec, uint32_t &grid, uint32_t &shift)
+static bool launch_geometry(const MultiTensorPlan &plan, int vec, int block, uint32_t &grid, uint32_t &shift)
 {
-    shift = slice_shift_for(plan.chunk_elements, vec);
+    shift = slice_shift_for(plan.chunk_elements, vec, block);
     const uint64_t blocks = (uint64_t)plan.num_chunks << shift;
     if (blocks > 0x7FFFFFFFull) {
         set_error("parameter list needs %llu workgroups, more than one launch can address",
@@ -559,14 +560,14 @@ static bool launch_geometry(const MultiTensorPlan &plan, int vec, uint32_t &grid
     return true;
 }
 
-template <class Rule, int VEC>
+template <class Rule, int VEC, int BLOCK>
 static void launch_rule_vec(const Launch &l, const StepParams &prm, uint32_t grid, uint32_t shift)
 {
     if (current_nontemporal())
-        multi_tensor_update_kernel<Rule, VEC, true><<<grid, kBlock, 0, l.ctx->stream>>>(
+        multi_tensor_update_kernel<Rule, VEC, true, BLOCK><<<grid, BLOCK, 0, l.ctx->stream>>>(
             l.plan->d_chunks, shift, prm);
     else
-        multi_tensor_update_kernel<Rule, VEC, false><<<grid, kBlock, 0, l.ctx->stream>>>(
+        multi_tensor_update_kernel<Rule, VEC, false, BLOCK><<<grid, BLOCK, 0, l.ctx->stream>>>(
             l.plan->d_chunks, shift, prm);
 }
 
@@ -574,13 +575,21 @@ template <class Rule>
 static int launch_rule(const Launch &l, const StepParams &prm, int hip_error_code)
 {
     if (l.plan->num_chunks == 0) return 0;
-    int vec = current_vec();
-    if (vec == 0) vec = auto_vec(3 + 2 * Rule::NSTATE);   // w, g, states read; w, states written
+    constexpr int streams = 3 + 2 * Rule::NSTATE;          // w, g, states read; w, states written
+    int vec = current_vec(), block = current_block();
+    if (vec == 0) vec = auto_vec(streams);
+    if (block == 0) block = auto_block(streams);
     uint32_t grid, shift;
-    if (!launch_geometry(*l.plan, vec, grid, shift)) return hip_error_code;
-    if (vec == 4) launch_rule_vec<Rule, 4>(l, prm, grid, shift);
-    else if (vec == 2) launch_rule_vec<Rule, 2>(l, prm, grid, shift);
-    else launch_rule_vec<Rule, 1>(l, prm, grid, shift);
+    if (!launch_geometry(*l.plan, vec, block, grid, shift)) return hip_error_code;
+    if (block == 128) {
+        if (vec == 4) launch_rule_vec<Rule, 4, 128>(l, prm, grid, shift);
+        else if (vec == 2) launch_rule_vec<Rule, 2, 128>(l, prm, grid, shift);
+        else launch_rule_vec<Rule, 1, 128>(l, prm, grid, shift);
+    } else {
+        if (vec == 4) launch_rule_vec<Rule, 4, kBlock>(l, prm, grid, shift);
+        else if (vec == 2) launch_rule_vec<Rule, 2, kBlock>(l, prm, grid, shift);
+        else launch_rule_vec<Rule, 1, kBlock>(l, prm, grid, shift);
+    }
     return hip_ok(hipGetLastError(), "update kernel launch") ? 0 : hip_error_code;
 }
 
@@ -669,6 +678,13 @@ int gm_set_tuning(int chunk_elements, int nontemporal, int vec)
     return 0;
 }
 
+int gm_set_workgroup_lanes(int lanes)
+{
+    if (lanes != 0 && lanes != 128 && lanes != kBlock) return -1;
+    g_block.store(lanes);
+    return 0;
+}
+
 int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                               uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
                               int num_weights, int *buffer_sizes, float learning_rate,
@@ -696,13 +712,18 @@ int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     int vec = current_vec();
     if (vec == 0) vec = auto_vec(5);
     const bool nt = current_nontemporal();
+    int block = current_block();
+    if (block == 0) block = auto_block(5);
     uint32_t grid, shift;
-    if (!launch_geometry(*l.plan, vec, grid, shift)) return -10;
+    if (!launch_geometry(*l.plan, vec, block, grid, shift)) return -10;
     hipStream_t st = l.ctx->stream;
-#define GM_LAUNCH_SGD(V, N) multi_tensor_sgd_kernel<V, N><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, shift, p)
-    if (vec == 4) { if (nt) GM_LAUNCH_SGD(4, true); else GM_LAUNCH_SGD(4, false); }
-    else if (vec == 2) { if (nt) GM_LAUNCH_SGD(2, true); else GM_LAUNCH_SGD(2, false); }
-    else { if (nt) GM_LAUNCH_SGD(1, true); else GM_LAUNCH_SGD(1, false); }
+#define GM_LAUNCH_SGD(V, N, B) multi_tensor_sgd_kernel<V, N, B><<<grid, B, 0, st>>>(l.plan->d_chunks, shift, p)
+#define GM_LAUNCH_SGD_B(B)                                                              \
+    if (vec == 4) { if (nt) GM_LAUNCH_SGD(4, true, B); else GM_LAUNCH_SGD(4, false, B); }        \
+    else if (vec == 2) { if (nt) GM_LAUNCH_SGD(2, true, B); else GM_LAUNCH_SGD(2, false, B); }   \
+    else { if (nt) GM_LAUNCH_SGD(1, true, B); else GM_LAUNCH_SGD(1, false, B); }
+    if (block == 128) { GM_LAUNCH_SGD_B(128) } else { GM_LAUNCH_SGD_B(kBlock) }
+#undef GM_LAUNCH_SGD_B
 #undef GM_LAUNCH_SGD
     return hip_ok(hipGetLastError(), "sgd kernel launch") ? 0 : -10;
 }
@@ -1035,8 +1056,8 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
                        uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
                        uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
                        int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
-                       float weight_decay, int step_count, bool async, AmpDeviceState *host_mirror,
-                       Launch &l, std::unique_lock<std::mutex> &lock)
+                       float weight_decay, int step_count, bool async, Launch &l,
+                       std::unique_lock<std::mutex> &lock)
 {
     PlanRequest req{};
     req.kind = kRuleAdamAMP;
@@ -1065,9 +1086,14 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     p.eps = epsilon;
     p.weight_decay = weight_decay;
 
+    // The context lock is held from here on: the issue counters of the loss-scale state are
+    // only read and advanced under it.  An asynchronous step's post-state goes into the ring
+    // slot of its issue number, a synchronous step's into slot 0.
+    AmpDeviceState *host_mirror = amp->h_pinned;
     AmpBiasTable bias{};
     if (async) {
         if (!amp_poll(amp, true)) return -6;
+        host_mirror = &amp->h_pinned[1 + (amp->issued + 1) % kAmpMaxInFlight];
         const int in_flight = (int)(amp->issued - amp->confirmed_issue);
         if (in_flight > amp->max_in_flight) amp->max_in_flight = in_flight;
         bias.base = amp->confirmed_applied;
@@ -1085,14 +1111,19 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
         int vec = current_vec();
         if (vec == 0) vec = auto_vec(8);
         const bool nt = current_nontemporal();
+        int block = current_block();
+        if (block == 0) block = auto_block(8);
         uint32_t grid, shift;
-        if (!launch_geometry(*l.plan, vec, grid, shift)) return -6;
+        if (!launch_geometry(*l.plan, vec, block, grid, shift)) return -6;
         if (nt) amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
         else amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
-#define GM_LAUNCH_AMP(V, N) amp_adam_update_kernel<V, N><<<grid, kBlock, 0, st>>>(l.plan->d_chunks, shift, p, amp->d_state, bias)
-        if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true); else GM_LAUNCH_AMP(4, false); }
-        else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true); else GM_LAUNCH_AMP(2, false); }
-        else { if (nt) GM_LAUNCH_AMP(1, true); else GM_LAUNCH_AMP(1, false); }
+#define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<grid, B, 0, st>>>(l.plan->d_chunks, shift, p, amp->d_state, bias)
+#define GM_LAUNCH_AMP_B(B)                                                              \
+        if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true, B); else GM_LAUNCH_AMP(4, false, B); }        \
+        else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true, B); else GM_LAUNCH_AMP(2, false, B); }   \
+        else { if (nt) GM_LAUNCH_AMP(1, true, B); else GM_LAUNCH_AMP(1, false, B); }
+        if (block == 128) { GM_LAUNCH_AMP_B(128) } else { GM_LAUNCH_AMP_B(kBlock) }
+#undef GM_LAUNCH_AMP_B
 #undef GM_LAUNCH_AMP
     }
     amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror);
@@ -1114,7 +1145,7 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
     std::unique_lock<std::mutex> lock;
     if (int rc = amp_enqueue(device, amp, weight_buffers, gradient16_buffers, momentum_buffers,
                              variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
-                             beta1, beta2, epsilon, weight_decay, step_count, false, amp->h_pinned, l, lock))
+                             beta1, beta2, epsilon, weight_decay, step_count, false, l, lock))
         return rc;
     if (!hip_ok(hipStreamSynchronize(l.ctx->stream), "hipStreamSynchronize")) return -6;
     amp->confirmed_issue = amp->issued;
@@ -1136,13 +1167,13 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
     if (!amp) return -16;
     Launch l{};
     std::unique_lock<std::mutex> lock;
-    // the post-state of this step goes into its ring slot; the event marks its arrival
-    const uint64_t issue = amp->issued + 1;
-    const int slot = (int)(issue % kAmpMaxInFlight);
     if (int rc = amp_enqueue(device, amp, weight_buffers, gradient16_buffers, momentum_buffers,
                              variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
-                             beta1, beta2, epsilon, weight_decay, 0, true, &amp->h_pinned[1 + slot], l, lock))
+                             beta1, beta2, epsilon, weight_decay, 0, true, l, lock))
         return rc;
+    // the event marks the arrival of this step's post-state in its ring slot
+    const uint64_t issue = amp->issued + 1;
+    const int slot = (int)(issue % kAmpMaxInFlight);
     if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
         // the step itself is enqueued; resynchronise the bookkeeping with the device
         (void)amp_download(amp);

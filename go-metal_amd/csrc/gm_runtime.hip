@@ -100,75 +100,89 @@ uint64_t registry_generation() { return g_reg_generation.load(); }
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
-// fp32 -> fp16, round to nearest even (v_cvt_f16_f32); 4 elements per lane,
-// scalar tail.
-__global__ void __launch_bounds__(256)
-convert_f32_to_f16_kernel(const float *__restrict__ src, __half *__restrict__ dst, size_t n)
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+#define GM_GLOBAL __attribute__((address_space(1)))
+
+// Launch shapes of the kernels below, measured on MI355X over 2^28 elements (1 GiB of fp32): with one
+// or two streams the memory system prefers 16-byte accesses from single-wavefront workgroups, the
+// opposite of the seven-stream optimizer update.  Conversion: 4 elements per lane (16-byte side +
+// 8-byte side, non-temporal), 64 lanes: 85-87 % of the 8 TB/s peak, against 75-78 % for a grid-stride
+// loop of 256-lane workgroups and 35-60 % for 1 or 2 elements per lane.  Copy: one 16-byte vector per
+// lane, 64 lanes, 83 % (hipMemcpyAsync device-to-device: 63 %).  Zero fill: one 16-byte store per
+// lane, 256 lanes, ordinary stores, 85 % (64 lanes: 59 %; grid-stride loop: 74 %).
+constexpr int kConvertBlock = 64;
+constexpr int kCopyBlock = 64;
+constexpr int kZeroBlock = 256;
+
+// fp32 -> fp16, round to nearest even (v_cvt_f16_f32).  GROUPED: lane i converts elements
+// [4 i, 4 i + 4); the last n % 4 elements go to the first lanes of workgroup 0.  Otherwise
+// (a view that is not aligned for 16-byte / 8-byte accesses) one element per lane.
+template <bool GROUPED>
+__global__ void __launch_bounds__(kConvertBlock)
+convert_f32_to_f16_kernel(const float *__restrict__ src, _Float16 *__restrict__ dst, size_t n)
 {
-    // 4-element groups only when both views are aligned for them (handles may be offset addresses)
-    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 8 == 0;
-    const size_t n4 = aligned ? n / 4 : 0;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-        floatx4 x = reinterpret_cast<const floatx4 *>(src)[i];
-        __half2 lo = __halves2half2(__float2half_rn(x.x), __float2half_rn(x.y));
-        __half2 hi = __halves2half2(__float2half_rn(x.z), __float2half_rn(x.w));
-        uint2 packed;
-        packed.x = *reinterpret_cast<unsigned int *>(&lo);
-        packed.y = *reinterpret_cast<unsigned int *>(&hi);
-        reinterpret_cast<uint2 *>(dst)[i] = packed;
+    const size_t i = (size_t)blockIdx.x * kConvertBlock + threadIdx.x;
+    if (!GROUPED) {
+        if (i < n) dst[i] = (_Float16)src[i];
+        return;
     }
-    for (size_t i = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-        dst[i] = __float2half_rn(src[i]);
+    const size_t n4 = n / 4;
+    if (i < n4) {
+        const floatx4 x = __builtin_nontemporal_load(((const GM_GLOBAL floatx4 *)(src)) + i);
+        halfx4 y;
+#pragma unroll
+        for (int c = 0; c < 4; c++) y[c] = (_Float16)x[c];
+        __builtin_nontemporal_store(y, ((GM_GLOBAL halfx4 *)(dst)) + i);
+    }
+    if (blockIdx.x == 0 && n4 * 4 + threadIdx.x < n) dst[n4 * 4 + threadIdx.x] = (_Float16)src[n4 * 4 + threadIdx.x];
 }
 
-__global__ void __launch_bounds__(256)
-convert_f16_to_f32_kernel(const __half *__restrict__ src, float *__restrict__ dst, size_t n)
+template <bool GROUPED>
+__global__ void __launch_bounds__(kConvertBlock)
+convert_f16_to_f32_kernel(const _Float16 *__restrict__ src, float *__restrict__ dst, size_t n)
 {
-    const bool aligned = reinterpret_cast<uintptr_t>(src) % 8 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
-    const size_t n4 = aligned ? n / 4 : 0;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-        uint2 packed = reinterpret_cast<const uint2 *>(src)[i];
-        __half2 lo = *reinterpret_cast<__half2 *>(&packed.x);
-        __half2 hi = *reinterpret_cast<__half2 *>(&packed.y);
+    const size_t i = (size_t)blockIdx.x * kConvertBlock + threadIdx.x;
+    if (!GROUPED) {
+        if (i < n) dst[i] = (float)src[i];
+        return;
+    }
+    const size_t n4 = n / 4;
+    if (i < n4) {
+        const halfx4 x = __builtin_nontemporal_load(((const GM_GLOBAL halfx4 *)(src)) + i);
         floatx4 y;
-        y.x = __low2float(lo);
-        y.y = __high2float(lo);
-        y.z = __low2float(hi);
-        y.w = __high2float(hi);
-        reinterpret_cast<floatx4 *>(dst)[i] = y;
+#pragma unroll
+        for (int c = 0; c < 4; c++) y[c] = (float)x[c];
+        __builtin_nontemporal_store(y, ((GM_GLOBAL floatx4 *)(dst)) + i);
     }
-    for (size_t i = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-        dst[i] = __half2float(src[i]);
+    if (blockIdx.x == 0 && n4 * 4 + threadIdx.x < n) dst[n4 * 4 + threadIdx.x] = (float)src[n4 * 4 + threadIdx.x];
 }
 
-// Zero fill: 16-byte stores, byte tail.  (A kernel rather than hipMemsetAsync, so
-// the entry point stays safe to record into a HIP graph.)
-__global__ void __launch_bounds__(256)
-zero_kernel(unsigned char *__restrict__ dst, size_t bytes)
+// Zero fill: bytes up to the first 16-byte boundary and after the last one by workgroup 0, one
+// 16-byte store per lane between them.  (A kernel rather than hipMemsetAsync, so the entry point
+// stays safe to record into a HIP graph.)
+__global__ void __launch_bounds__(kZeroBlock)
+zero_kernel(unsigned char *__restrict__ dst, size_t bytes, size_t head, size_t n16)
 {
-    // bytes up to the first 16-byte boundary, 16-byte stores, byte tail
-    size_t head = (16 - reinterpret_cast<uintptr_t>(dst) % 16) % 16;
-    if (head > bytes) head = bytes;
-    const size_t n16 = (bytes - head) / 16;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t i = (size_t)blockIdx.x * kZeroBlock + threadIdx.x;
     const uintx4 z = {0u, 0u, 0u, 0u};
-    for (size_t i = tid; i < n16; i += stride) reinterpret_cast<uintx4 *>(dst + head)[i] = z;
+    if (i < n16) ((GM_GLOBAL uintx4 *)(dst + head))[i] = z;
     if (blockIdx.x == 0) {
-        for (size_t i = threadIdx.x; i < head; i += blockDim.x) dst[i] = 0;
-        for (size_t i = head + n16 * 16 + threadIdx.x; i < bytes; i += blockDim.x) dst[i] = 0;
+        for (size_t k = threadIdx.x; k < head; k += kZeroBlock) dst[k] = 0;
+        for (size_t k = head + n16 * 16 + threadIdx.x; k < bytes; k += kZeroBlock) dst[k] = 0;
     }
 }
 
-// Plain copy, one 16-byte vector per lane, one wavefront per workgroup: the
-// fastest copy shape measured on MI355X (about 6.8 TB/s read + write).
-__global__ void __launch_bounds__(64)
-copy_probe_kernel(const uintx4 *__restrict__ src, uintx4 *__restrict__ dst, size_t n16)
+// Plain copy, one 16-byte vector per lane, one wavefront per workgroup; the last bytes % 16 bytes
+// go to the first lanes of workgroup 0.  Both addresses are 16-byte aligned.
+__global__ void __launch_bounds__(kCopyBlock)
+copy_kernel(const unsigned char *__restrict__ src, unsigned char *__restrict__ dst, size_t bytes)
 {
-    const size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
-    if (i < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
+    const size_t n16 = bytes / 16;
+    const size_t i = (size_t)blockIdx.x * kCopyBlock + threadIdx.x;
+    if (i < n16)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(((const GM_GLOBAL uintx4 *)(src)) + i),
+                                    ((GM_GLOBAL uintx4 *)(dst)) + i);
+    if (blockIdx.x == 0 && n16 * 16 + threadIdx.x < bytes) dst[n16 * 16 + threadIdx.x] = src[n16 * 16 + threadIdx.x];
 }
 
 __device__ inline uint64_t splitmix64(uint64_t x)
@@ -309,8 +323,12 @@ int zero_metal_buffer(uintptr_t device, uintptr_t buffer, int size)
         set_error("zero of %d bytes exceeds the %zu-byte buffer", size, len);
         return -5;
     }
-    const unsigned int grid = grid_for(((size_t)size + 15) / 16, 256, 1u << 16);
-    zero_kernel<<<grid, 256, 0, ctx->stream>>>(reinterpret_cast<unsigned char *>(buffer), (size_t)size);
+    size_t head = (16 - buffer % 16) % 16;
+    if (head > (size_t)size) head = (size_t)size;
+    const size_t n16 = ((size_t)size - head) / 16;
+    const unsigned int grid = grid_for(n16, kZeroBlock, 0x7FFFFFFFu);
+    zero_kernel<<<grid, kZeroBlock, 0, ctx->stream>>>(reinterpret_cast<unsigned char *>(buffer), (size_t)size, head,
+                                                      n16);
     if (!hip_ok(hipGetLastError(), "zero kernel launch")) return -5;
     return 0;
 }
@@ -404,13 +422,22 @@ int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, 
                   dst_len);
         return -5;
     }
-    const unsigned int grid = grid_for((total + 3) / 4, 256, 1u << 20);
-    if (to_half)
-        convert_f32_to_f16_kernel<<<grid, 256, 0, ctx->stream>>>(
-            reinterpret_cast<const float *>(src_buffer), reinterpret_cast<__half *>(dst_buffer), total);
-    else
-        convert_f16_to_f32_kernel<<<grid, 256, 0, ctx->stream>>>(
-            reinterpret_cast<const __half *>(src_buffer), reinterpret_cast<float *>(dst_buffer), total);
+    // 4-element groups only when both views are aligned for them (handles may be offset addresses)
+    const bool grouped = src_buffer % (to_half ? 16 : 8) == 0 && dst_buffer % (to_half ? 8 : 16) == 0;
+    const size_t lanes = grouped ? (total / 4 > 0 ? total / 4 : 1) : total;
+    if ((lanes + kConvertBlock - 1) / kConvertBlock > 0x7FFFFFFFull) {
+        set_error("conversion of %zu elements needs more workgroups than one launch can address", total);
+        return -5;
+    }
+    const unsigned int grid = grid_for(lanes, kConvertBlock, 0x7FFFFFFFu);
+    const float *f_src = reinterpret_cast<const float *>(src_buffer);
+    const _Float16 *h_src = reinterpret_cast<const _Float16 *>(src_buffer);
+    float *f_dst = reinterpret_cast<float *>(dst_buffer);
+    _Float16 *h_dst = reinterpret_cast<_Float16 *>(dst_buffer);
+    if (to_half && grouped) convert_f32_to_f16_kernel<true><<<grid, kConvertBlock, 0, ctx->stream>>>(f_src, h_dst, total);
+    else if (to_half) convert_f32_to_f16_kernel<false><<<grid, kConvertBlock, 0, ctx->stream>>>(f_src, h_dst, total);
+    else if (grouped) convert_f16_to_f32_kernel<true><<<grid, kConvertBlock, 0, ctx->stream>>>(h_src, f_dst, total);
+    else convert_f16_to_f32_kernel<false><<<grid, kConvertBlock, 0, ctx->stream>>>(h_src, f_dst, total);
     if (!hip_ok(hipGetLastError(), "convert kernel launch")) return -4;
     return 0;
 }
@@ -426,11 +453,19 @@ int copy_buffer_to_buffer_sync(uintptr_t src_buffer, uintptr_t dst_buffer, int s
     if (dst_len != 0 && (size_t)dst_offset + (size_t)size > dst_len) return -5;
     Context *ctx = default_context();
     if (!ctx || !make_current(ctx)) return -10;
-    if (!hip_ok(hipMemcpyAsync(reinterpret_cast<char *>(dst_buffer) + dst_offset,
-                               reinterpret_cast<const char *>(src_buffer) + src_offset, (size_t)size,
-                               hipMemcpyDeviceToDevice, ctx->stream), "hipMemcpyAsync(D2D)") ||
-        !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
+    const uintptr_t from = src_buffer + (uintptr_t)src_offset, to = dst_buffer + (uintptr_t)dst_offset;
+    const bool overlap = from < to + (uintptr_t)size && to < from + (uintptr_t)size;
+    if (from % 16 == 0 && to % 16 == 0 && !overlap) {
+        // the library's own copy kernel: faster than the runtime's device-to-device copy
+        const unsigned int grid = grid_for((size_t)size / 16, kCopyBlock, 0x7FFFFFFFu);
+        copy_kernel<<<grid, kCopyBlock, 0, ctx->stream>>>(reinterpret_cast<const unsigned char *>(from),
+                                                          reinterpret_cast<unsigned char *>(to), (size_t)size);
+        if (!hip_ok(hipGetLastError(), "copy kernel launch")) return -10;
+    } else if (!hip_ok(hipMemcpyAsync(reinterpret_cast<void *>(to), reinterpret_cast<const void *>(from),
+                                      (size_t)size, hipMemcpyDeviceToDevice, ctx->stream), "hipMemcpyAsync(D2D)")) {
         return -10;
+    }
+    if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize")) return -10;
     return 0;
 }
 
@@ -542,10 +577,10 @@ int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, 
     }
     const size_t n16 = bytes / 16;
     if (n16 == 0) return 0;
-    const size_t blocks = (n16 + 63) / 64;
+    const size_t blocks = (n16 + kCopyBlock - 1) / kCopyBlock;
     if (blocks > 0x7FFFFFFFull) return -5;
-    copy_probe_kernel<<<(unsigned int)blocks, 64, 0, ctx->stream>>>(
-        reinterpret_cast<const uintx4 *>(src_buffer), reinterpret_cast<uintx4 *>(dst_buffer), n16);
+    copy_kernel<<<(unsigned int)blocks, kCopyBlock, 0, ctx->stream>>>(
+        reinterpret_cast<const unsigned char *>(src_buffer), reinterpret_cast<unsigned char *>(dst_buffer), bytes);
     return hip_ok(hipGetLastError(), "copy probe launch") ? 0 : -10;
 }
 

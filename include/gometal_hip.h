@@ -325,6 +325,9 @@ int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, 
  * with up to five streams, else 1).
  * -1 if the combination is not valid (nothing changes). */
 int gm_set_tuning(int chunk_elements, int nontemporal, int vec);
+/* Lanes per workgroup of the update kernels: 128 or 256; 0 = default (128 for rules with up to
+ * five streams, else 256).  -1 on any other value (nothing changes). */
+int gm_set_workgroup_lanes(int lanes);
 
 #ifdef __cplusplus
 }

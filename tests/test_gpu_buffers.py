@@ -176,6 +176,62 @@ def test_offset_views_take_the_unaligned_paths(dev):
         dev.free(h)
 
 
+@pytest.mark.parametrize("src_off,dst_off,size", [
+    (0, 0, 4096), (0, 0, 4099), (16, 48, 1000), (16, 48, 7),          # 16-byte aligned: the library's copy kernel
+    (4, 8, 4096), (1, 3, 333), (16, 5, 64),                            # unaligned: the runtime's copy
+    (0, 0, 16 * 64 * 3 + 5), (32, 16, 16 * 64),                        # several workgroups, exact multiple
+])
+def test_buffer_to_buffer_copy_offsets_sizes_and_canaries(dev, src_off, dst_off, size):
+    """Every (offset, size) class of copy_buffer_to_buffer_sync moves exactly the bytes asked for."""
+    total = 8192
+    rng = np.random.default_rng(size)
+    a = rng.integers(0, 256, total, dtype=np.uint8)
+    b = rng.integers(0, 256, total, dtype=np.uint8)
+    src, dst = dev.from_numpy(a), dev.from_numpy(b)
+    assert dev.lib.copy_buffer_to_buffer_sync(src, dst, src_off, dst_off, size) == 0
+    want = b.copy()
+    want[dst_off:dst_off + size] = a[src_off:src_off + size]
+    assert np.array_equal(dev.to_numpy(dst, total, np.uint8), want)
+    assert np.array_equal(dev.to_numpy(src, total, np.uint8), a)
+    dev.free(src)
+    dev.free(dst)
+
+
+def test_buffer_to_buffer_copy_inside_one_buffer(dev):
+    """Disjoint ranges of one buffer copy exactly; overlapping ranges go to the runtime's copy and at
+    least return without error (their result is unspecified in the reference as well)."""
+    a = np.random.default_rng(11).integers(0, 256, 4096, dtype=np.uint8)
+    buf = dev.from_numpy(a)
+    assert dev.lib.copy_buffer_to_buffer_sync(buf, buf, 0, 2048, 1024) == 0
+    want = a.copy()
+    want[2048:3072] = a[:1024]
+    assert np.array_equal(dev.to_numpy(buf, 4096, np.uint8), want)
+    assert dev.lib.copy_buffer_to_buffer_sync(buf, buf, 0, 16, 1024) == 0
+    dev.free(buf)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 63, 64, 255, 256, 257, 1027, 65537])
+def test_convert_lengths_around_the_group_and_workgroup_sizes(dev, n):
+    """Conversions work in 4-element groups, 64 lanes to a workgroup, with the last n % 4 elements apart:
+    every length class, with canaries behind the destination."""
+    o = oracle()
+    x = (np.random.default_rng(n).standard_normal(n) * 100).astype(np.float32)
+    src = dev.from_numpy(x)
+    half = dev.from_numpy(np.full(n + 8, 0x5555, np.uint16))
+    shape = (ctypes.c_int * 1)(n)
+    assert dev.lib.convert_tensor_type(src, half, shape, 1, 0, 2, dev.handle) == 0
+    got = dev.to_numpy(half, n + 8, np.uint16)
+    want = o.f32_to_f16(x)
+    assert np.array_equal(got[:n], want) and np.all(got[n:] == 0x5555)
+    back = dev.from_numpy(np.full(n + 4, -3.0, np.float32))
+    assert dev.lib.convert_tensor_type(half, back, shape, 1, 2, 0, dev.handle) == 0
+    got32 = dev.to_numpy(back, n + 4)
+    assert np.array_equal(got32[:n].view(np.uint32), o.f16_to_f32(want).view(np.uint32))
+    assert np.all(got32[n:] == -3.0)
+    for h in (src, half, back):
+        dev.free(h)
+
+
 def test_ranges_beyond_an_allocation_are_refused(dev):
     """The reference trusts its callers here; an overrun on a GPU is a fault, so buffers of this
     library are checked against their recorded length."""
