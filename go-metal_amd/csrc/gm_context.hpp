@@ -18,6 +18,10 @@ namespace gm {
 
 void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 void clear_error();
+// For the catch (...) block of an entry point: records the exception in flight as the thread's
+// last error.  No exception may cross the C boundary; the entry point then returns the code the
+// reference returns from its own @catch block.
+void note_exception() noexcept;
 
 // true when the HIP call succeeded; otherwise records "what: <hip error>".
 bool hip_ok(hipError_t e, const char *what);

@@ -626,7 +626,7 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uin
                                 int history_index, float initial_step, float c1, float c2,
                                 int max_line_search, float current_loss, float prev_loss,
                                 float *step_size)
-{
+try {
     // The reference performs no line search: the Wolfe constants and the losses are accepted
     // and ignored (bridge_optimizer.m:1231-1233).
     (void)c1; (void)c2; (void)max_line_search; (void)current_loss; (void)prev_loss;
@@ -739,6 +739,9 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uin
         launch_reduction(ctx, p, Epilogue{kOpRho, nullptr, nullptr, rho_ptr(prev), p.d_scalars});
     }
     return hip_ok(hipGetLastError(), "L-BFGS kernel launch") ? 0 : -8;
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
@@ -762,7 +765,7 @@ int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffe
 
 int gm_lbfgs_dot(uintptr_t device, uintptr_t *a_buffers, uintptr_t *b_buffers, int num_tensors,
                  int *buffer_sizes, float *result)
-{
+try {
     Entry en;
     if (int rc = enter(device, buffer_sizes, num_tensors, en)) return rc;
     if (!a_buffers || !b_buffers || !result) {
@@ -812,6 +815,9 @@ int gm_lbfgs_dot(uintptr_t device, uintptr_t *a_buffers, uintptr_t *b_buffers, i
     if (d_rows) (void)hipFree(d_rows);
     if (h_result) (void)hipHostFree(h_result);
     return rc;
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 }  // extern "C"

@@ -689,7 +689,7 @@ int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                               uintptr_t *gradient_buffers, uintptr_t *momentum_buffers,
                               int num_weights, int *buffer_sizes, float learning_rate,
                               float momentum, float weight_decay, int nesterov, int step_count)
-{
+try {
     (void)step_count;   // unused by the reference as well
     PlanRequest req{};
     req.kind = kRuleSGD;
@@ -726,6 +726,9 @@ int execute_sgd_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
 #undef GM_LAUNCH_SGD_B
 #undef GM_LAUNCH_SGD
     return hip_ok(hipGetLastError(), "sgd kernel launch") ? 0 : -10;
+} catch (...) {
+    note_exception();
+    return -10;
 }
 
 int execute_adam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
@@ -733,10 +736,13 @@ int execute_adam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                uintptr_t *variance_buffers, int num_weights, int *buffer_sizes,
                                float learning_rate, float beta1, float beta2, float epsilon,
                                float weight_decay, int step_count)
-{
+try {
     return adam_like_step(kRuleAdam, device, weight_buffers, gradient_buffers, momentum_buffers,
                           variance_buffers, num_weights, buffer_sizes, learning_rate, beta1, beta2,
                           epsilon, weight_decay, step_count);
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 int execute_adam_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
@@ -745,12 +751,15 @@ int execute_adam_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffer
                                       int *buffer_sizes, float learning_rate, float beta1,
                                       float beta2, float epsilon, float weight_decay,
                                       int step_count, uintptr_t command_pool)
-{
+try {
     if (device == 0) return -1;
     if (command_pool == 0) return -15;
     return adam_like_step(kRuleAdam, device, weight_buffers, gradient_buffers, momentum_buffers,
                           variance_buffers, num_weights, buffer_sizes, learning_rate, beta1, beta2,
                           epsilon, weight_decay, step_count);
+} catch (...) {
+    note_exception();
+    return -13;
 }
 
 int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
@@ -758,10 +767,13 @@ int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                 uintptr_t *variance_buffers, int num_weights, int *buffer_sizes,
                                 float learning_rate, float beta1, float beta2, float epsilon,
                                 float weight_decay, int step_count)
-{
+try {
     return adam_like_step(kRuleNAdam, device, weight_buffers, gradient_buffers, momentum_buffers,
                           variance_buffers, num_weights, buffer_sizes, learning_rate, beta1, beta2,
                           epsilon, weight_decay, step_count);
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 int execute_rmsprop_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
@@ -771,7 +783,7 @@ int execute_rmsprop_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                   int num_weights, int *buffer_sizes, float learning_rate,
                                   float alpha, float epsilon, float weight_decay, float momentum,
                                   bool centered, int step_count)
-{
+try {
     (void)step_count;
     const bool use_momentum = momentum > 0.0f;
     PlanRequest req{};
@@ -804,6 +816,9 @@ int execute_rmsprop_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     if (use_momentum) return launch_rule<RmsPropRule<true, false>>(l, p, -8);
     if (centered) return launch_rule<RmsPropRule<false, true>>(l, p, -8);
     return launch_rule<RmsPropRule<false, false>>(l, p, -8);
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 int execute_adagrad_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
@@ -811,7 +826,7 @@ int execute_adagrad_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                   uintptr_t *squared_grad_avg_buffers, int num_weights,
                                   int *buffer_sizes, float learning_rate, float epsilon,
                                   float weight_decay)
-{
+try {
     PlanRequest req{};
     req.kind = kRuleAdaGrad;
     req.num_tensors = num_weights;
@@ -828,6 +843,9 @@ int execute_adagrad_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     p.eps = epsilon;
     p.weight_decay = weight_decay;
     return launch_rule<AdaGradRule>(l, p, -8);
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 int execute_adagrad_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
@@ -835,11 +853,14 @@ int execute_adagrad_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buf
                                          uintptr_t *squared_grad_avg_buffers, int num_weights,
                                          int *buffer_sizes, float learning_rate, float epsilon,
                                          float weight_decay, uintptr_t command_pool)
-{
+try {
     (void)command_pool;
     return execute_adagrad_step_mpsgraph(device, weight_buffers, gradient_buffers,
                                          squared_grad_avg_buffers, num_weights, buffer_sizes,
                                          learning_rate, epsilon, weight_decay);
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 int execute_adadelta_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
@@ -847,7 +868,7 @@ int execute_adadelta_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                    uintptr_t *squared_grad_avg_buffers,
                                    uintptr_t *squared_update_avg_buffers, int num_weights,
                                    int *buffer_sizes, float rho, float epsilon, float weight_decay)
-{
+try {
     PlanRequest req{};
     req.kind = kRuleAdaDelta;
     req.num_tensors = num_weights;
@@ -867,6 +888,9 @@ int execute_adadelta_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
     p.eps = epsilon;
     p.weight_decay = weight_decay;
     return launch_rule<AdaDeltaRule>(l, p, -8);
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 int execute_adadelta_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
@@ -875,11 +899,14 @@ int execute_adadelta_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_bu
                                           uintptr_t *squared_update_avg_buffers, int num_weights,
                                           int *buffer_sizes, float rho, float epsilon,
                                           float weight_decay, uintptr_t command_pool)
-{
+try {
     (void)command_pool;
     return execute_adadelta_step_mpsgraph(device, weight_buffers, gradient_buffers,
                                           squared_grad_avg_buffers, squared_update_avg_buffers,
                                           num_weights, buffer_sizes, rho, epsilon, weight_decay);
+} catch (...) {
+    note_exception();
+    return -8;
 }
 
 // ---------------------------------------------------------- mixed precision --
@@ -959,7 +986,7 @@ static void amp_free(AmpState *s)
 
 uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_factor,
                               float backoff_factor, int growth_interval)
-{
+try {
     clear_error();
     if (device == 0) return 0;
     Context *ctx = resolve_device(device);
@@ -987,15 +1014,20 @@ uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_f
         return 0;
     }
     return reinterpret_cast<uintptr_t>(s);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void gm_amp_state_destroy(uintptr_t amp_state)
-{
+try {
     AmpState *s = amp_from_handle(amp_state);
     if (!s) return;
     make_current(s->ctx);
     (void)hipStreamSynchronize(s->ctx->stream);     // ring copies may still be in flight
     amp_free(s);
+} catch (...) {
+    note_exception();
 }
 
 int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker)
@@ -1005,7 +1037,7 @@ int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker)
 
 int gm_amp_state_query(uintptr_t amp_state, float *scale, int *growth_tracker, int *applied_steps,
                        int *skipped_steps)
-{
+try {
     AmpState *s = amp_from_handle(amp_state);
     if (!s) return -16;
     if (!make_current(s->ctx)) return -6;
@@ -1016,6 +1048,9 @@ int gm_amp_state_query(uintptr_t amp_state, float *scale, int *growth_tracker, i
     if (applied_steps) *applied_steps = s->h_pinned->applied_steps;
     if (skipped_steps) *skipped_steps = s->h_pinned->skipped_steps;
     return 0;
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 int gm_amp_state_max_in_flight(uintptr_t amp_state)
@@ -1025,7 +1060,7 @@ int gm_amp_state_max_in_flight(uintptr_t amp_state)
 }
 
 int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
-{
+try {
     AmpState *s = amp_from_handle(amp_state);
     if (!s) return -16;
     if (!make_current(s->ctx)) return -6;
@@ -1035,10 +1070,13 @@ int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
     s->h_pinned->inv_scale = 1.0f / scale;
     s->h_pinned->growth_tracker = growth_tracker;
     return amp_upload(s) ? 0 : -6;
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 int gm_amp_state_set_step_count(uintptr_t amp_state, int applied_steps)
-{
+try {
     AmpState *s = amp_from_handle(amp_state);
     if (!s) return -16;
     if (applied_steps < 0) return -5;
@@ -1049,6 +1087,9 @@ int gm_amp_state_set_step_count(uintptr_t amp_state, int applied_steps)
     if (!amp_upload(s)) return -6;
     s->confirmed_applied = applied_steps;
     return 0;
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 // Plan, parameters and the three launches shared by the synchronous and the asynchronous step.
@@ -1137,7 +1178,7 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
                           float beta2, float epsilon, float weight_decay, int step_count,
                           uintptr_t amp_state, int *skipped, float *scale_out,
                           int *growth_tracker_out)
-{
+try {
     if (device == 0) return -1;
     AmpState *amp = amp_from_handle(amp_state);
     if (!amp) return -16;
@@ -1154,6 +1195,9 @@ int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
     if (scale_out) *scale_out = amp->h_pinned->scale;
     if (growth_tracker_out) *growth_tracker_out = amp->h_pinned->growth_tracker;
     return 0;
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
@@ -1161,7 +1205,7 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
                                 uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
                                 int num_weights, int *buffer_sizes, float learning_rate, float beta1,
                                 float beta2, float epsilon, float weight_decay, uintptr_t amp_state)
-{
+try {
     if (device == 0) return -1;
     AmpState *amp = amp_from_handle(amp_state);
     if (!amp) return -16;
@@ -1181,6 +1225,9 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
     }
     amp->issued = issue;
     return 0;
+} catch (...) {
+    note_exception();
+    return -6;
 }
 
 }  // extern "C"

@@ -9,6 +9,7 @@
 #include <hip/hip_fp16.h>
 
 #include <cstring>
+#include <exception>
 
 namespace gm {
 
@@ -24,6 +25,17 @@ void set_error(const char *fmt, ...)
 }
 
 void clear_error() { g_error[0] = '\0'; }
+
+void note_exception() noexcept
+{
+    try {
+        throw;
+    } catch (const std::exception &e) {
+        set_error("exception: %s", e.what());
+    } catch (...) {
+        set_error("unknown exception");
+    }
+}
 
 bool hip_ok(hipError_t e, const char *what)
 {
@@ -248,11 +260,14 @@ extern "C" {
 const char *gm_last_error(void) { return g_error; }
 
 uintptr_t create_metal_device(void)
-{
+try {
     Context *ctx = default_context();
     if (!ctx) return 0;
     ctx->refs.fetch_add(1);
     return reinterpret_cast<uintptr_t>(ctx);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void destroy_metal_device(uintptr_t device)
@@ -271,11 +286,14 @@ struct CommandQueue {
 static const uint64_t kQueueMagic = 0x676D5F7175657565ull;   // "gm_queue"
 
 uintptr_t create_command_queue(uintptr_t device)
-{
+try {
     if (device == 0) return 0;
     Context *ctx = resolve_device(device);
     if (!ctx) return 0;
     return reinterpret_cast<uintptr_t>(new CommandQueue{kQueueMagic, ctx});
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void release_command_queue(uintptr_t command_queue)
@@ -288,7 +306,7 @@ void release_command_queue(uintptr_t command_queue)
 }
 
 uintptr_t allocate_metal_buffer(uintptr_t device, int size, int device_type)
-{
+try {
     (void)device_type;
     if (device == 0 || size <= 0) return 0;
     Context *ctx = resolve_device(device);
@@ -298,22 +316,27 @@ uintptr_t allocate_metal_buffer(uintptr_t device, int size, int device_type)
     if (!hip_ok(hipMalloc(&p, aligned), "hipMalloc")) return 0;
     registry_add(reinterpret_cast<uintptr_t>(p), aligned);
     return reinterpret_cast<uintptr_t>(p);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void deallocate_metal_buffer(uintptr_t buffer)
-{
+try {
     if (buffer == 0) return;
     if (registry_length(buffer) == 0) return;   // not ours (or already freed): leave it alone
     registry_remove(buffer);
     Context *ctx = default_context();
     if (ctx) make_current(ctx);
     (void)hipFree(reinterpret_cast<void *>(buffer));   // hipFree waits for work in flight
+} catch (...) {
+    note_exception();
 }
 
 size_t gm_buffer_length(uintptr_t buffer) { return registry_length(buffer); }
 
 int zero_metal_buffer(uintptr_t device, uintptr_t buffer, int size)
-{
+try {
     if (device == 0 || buffer == 0) return -1;
     Context *ctx = resolve_device(device);
     if (!ctx || !make_current(ctx)) return -5;
@@ -331,6 +354,9 @@ int zero_metal_buffer(uintptr_t device, uintptr_t buffer, int size)
                                                       n16);
     if (!hip_ok(hipGetLastError(), "zero kernel launch")) return -5;
     return 0;
+} catch (...) {
+    note_exception();
+    return -5;
 }
 
 int zero_metal_buffer_mpsgraph(uintptr_t device, uintptr_t buffer, int size)
@@ -339,7 +365,7 @@ int zero_metal_buffer_mpsgraph(uintptr_t device, uintptr_t buffer, int size)
 }
 
 int copy_data_to_metal_buffer(uintptr_t buffer, void *data, int size)
-{
+try {
     if (buffer == 0 || data == nullptr || size <= 0) return -1;
     const size_t len = registry_length(buffer);
     if (len != 0 && (size_t)size > len) {
@@ -355,6 +381,9 @@ int copy_data_to_metal_buffer(uintptr_t buffer, void *data, int size)
         !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
         return -4;
     return 0;
+} catch (...) {
+    note_exception();
+    return -4;
 }
 
 int copy_float32_array_to_metal_buffer(uintptr_t buffer, float *data, int num_elements)
@@ -401,7 +430,7 @@ int copy_metal_buffer_to_int32_array(uintptr_t buffer, int *data, int num_elemen
 
 int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, int num_dims,
                         int src_type, int dst_type, uintptr_t device)
-{
+try {
     if (src_buffer == 0 || dst_buffer == 0 || shape == nullptr || num_dims <= 0) return -1;
     if (device == 0) return -2;
     size_t total = 1;
@@ -440,11 +469,14 @@ int convert_tensor_type(uintptr_t src_buffer, uintptr_t dst_buffer, int *shape, 
     else convert_f16_to_f32_kernel<false><<<grid, kConvertBlock, 0, ctx->stream>>>(h_src, f_dst, total);
     if (!hip_ok(hipGetLastError(), "convert kernel launch")) return -4;
     return 0;
+} catch (...) {
+    note_exception();
+    return -4;
 }
 
 int copy_buffer_to_buffer_sync(uintptr_t src_buffer, uintptr_t dst_buffer, int src_offset,
                                int dst_offset, int size)
-{
+try {
     if (src_buffer == 0 || dst_buffer == 0) return -1;
     if (size <= 0 || src_offset < 0 || dst_offset < 0) return -2;
     const size_t src_len = registry_length(src_buffer);
@@ -467,16 +499,22 @@ int copy_buffer_to_buffer_sync(uintptr_t src_buffer, uintptr_t dst_buffer, int s
     }
     if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize")) return -10;
     return 0;
+} catch (...) {
+    note_exception();
+    return -11;
 }
 
 int gm_synchronize(uintptr_t device)
-{
+try {
     if (device == 0) return -1;
     Context *ctx = resolve_device(device);
     if (!ctx) return -3;
     if (!make_current(ctx) || !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
         return -10;
     return 0;
+} catch (...) {
+    note_exception();
+    return -10;
 }
 
 // Cross-stream ordering without a host wait: an event recorded on one stream, waited for by
@@ -503,17 +541,20 @@ int gm_wait_for_stream(uintptr_t device, void *hip_stream) { return order_stream
 int gm_signal_stream(uintptr_t device, void *hip_stream) { return order_streams(device, hip_stream, false); }
 
 int gm_timer_start(uintptr_t device)
-{
+try {
     if (device == 0) return -1;
     Context *ctx = resolve_device(device);
     if (!ctx) return -3;
     if (!make_current(ctx) || !hip_ok(hipEventRecord(ctx->ev_start, ctx->stream), "hipEventRecord"))
         return -10;
     return 0;
+} catch (...) {
+    note_exception();
+    return -10;
 }
 
 float gm_timer_stop(uintptr_t device)
-{
+try {
     if (device == 0) return -1.0f;
     Context *ctx = resolve_device(device);
     if (!ctx || !make_current(ctx)) return -1.0f;
@@ -523,6 +564,9 @@ float gm_timer_stop(uintptr_t device)
         !hip_ok(hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop), "hipEventElapsedTime"))
         return -1.0f;
     return ms;
+} catch (...) {
+    note_exception();
+    return -1.0f;
 }
 
 static int fill_normal(uintptr_t device, uintptr_t buffer, size_t n, uint64_t seed, float mean,
@@ -562,7 +606,7 @@ int gm_fill_normal_f16(uintptr_t device, uintptr_t buffer, size_t num_elements, 
 }
 
 int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, size_t bytes)
-{
+try {
     if (device == 0) return -1;
     if (dst_buffer == 0 || src_buffer == 0) return -4;
     Context *ctx = resolve_device(device);
@@ -582,6 +626,9 @@ int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, 
     copy_kernel<<<(unsigned int)blocks, kCopyBlock, 0, ctx->stream>>>(
         reinterpret_cast<const unsigned char *>(src_buffer), reinterpret_cast<unsigned char *>(dst_buffer), bytes);
     return hip_ok(hipGetLastError(), "copy probe launch") ? 0 : -10;
+} catch (...) {
+    note_exception();
+    return -10;
 }
 
 }  // extern "C"

@@ -9,6 +9,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
 
 using namespace gometal;
 using namespace gometal::optimizer;
@@ -47,6 +48,23 @@ std::vector<Pointer> pointers(const uintptr_t *p, int n)
     return v;
 }
 
+// No exception may cross the C boundary (the caller is C, Go or Python): a failed allocation or a
+// standard-library error inside an entry point becomes that entry point's failure value, with the
+// reason in gmo_last_error().
+void note_exception() noexcept
+{
+    try {
+        try {
+            throw;
+        } catch (const std::exception &e) {
+            g_error = std::string("exception: ") + e.what();
+        } catch (...) {
+            g_error = "unknown exception";
+        }
+    } catch (...) {
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -55,31 +73,44 @@ const char *gmo_last_error(void) { return g_error.c_str(); }
 void gmo_free_string(char *s) { std::free(s); }
 
 uintptr_t gmo_memory_manager_new(uintptr_t device)
-{
+try {
     return reinterpret_cast<uintptr_t>(new memory::MemoryManager(reinterpret_cast<Pointer>(device)));
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void gmo_memory_manager_free(uintptr_t mm) { delete MM(mm); }
 
 void gmo_initialize_global_memory_manager(uintptr_t device)
-{
+try {
     memory::InitializeGlobalMemoryManager(reinterpret_cast<Pointer>(device));
+} catch (...) {
+    note_exception();
 }
 
 uintptr_t gmo_get_global_memory_manager(void)
-{
+try {
     return reinterpret_cast<uintptr_t>(memory::GetGlobalMemoryManager());
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 uintptr_t gmo_allocate_buffer(uintptr_t mm, int size)
-{
+try {
     if (!mm) return 0;
     return reinterpret_cast<uintptr_t>(MM(mm)->AllocateBuffer(size));
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void gmo_release_buffer(uintptr_t mm, uintptr_t buffer)
-{
+try {
     if (mm) MM(mm)->ReleaseBuffer(reinterpret_cast<Pointer>(buffer));
+} catch (...) {
+    note_exception();
 }
 
 int gmo_find_pool_size(uintptr_t mm, int size) { return mm ? MM(mm)->findPoolSize(size) : -1; }
@@ -88,7 +119,7 @@ int gmo_reference_max_pool_size(int buffer_size) { return memory::referenceMaxPo
 void gmo_set_pool_byte_budget(size_t bytes) { memory::SetPoolByteBudget(bytes); }
 
 int gmo_pool_stats(uintptr_t mm, int pool_size, int *available, int *allocated, int *max_size)
-{
+try {
     if (!mm) return -1;
     auto stats = MM(mm)->Stats();
     auto it = stats.find(memory::PoolKey{pool_size, memory::GPU});
@@ -99,10 +130,13 @@ int gmo_pool_stats(uintptr_t mm, int pool_size, int *available, int *allocated, 
     if (allocated) *allocated = b;
     if (max_size) *max_size = c;
     return 0;
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_default_config(int kind, float c[6])
-{
+try {
     switch (kind) {
     case GMO_SGD: {
         auto d = DefaultSGDConfig();
@@ -137,11 +171,14 @@ int gmo_default_config(int kind, float c[6])
     }
     }
     return -1;
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 uintptr_t gmo_optimizer_new(int kind, const float *c, const int *shape_dims, const int *shape_ndims,
                             int num_weights, uintptr_t memory_manager, uintptr_t device)
-{
+try {
     Shapes shapes;
     const int *d = shape_dims;
     for (int i = 0; i < num_weights; i++) {
@@ -185,35 +222,72 @@ uintptr_t gmo_optimizer_new(int kind, const float *c, const int *shape_dims, con
     }
     ok();
     return reinterpret_cast<uintptr_t>(new Handle{kind, std::move(opt)});
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void gmo_optimizer_free(uintptr_t opt) { delete H(opt); }
 
 int gmo_set_weight_buffers(uintptr_t opt, const uintptr_t *weight_buffers, int n)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     Error e = H(opt)->opt->SetWeightBuffers(pointers(weight_buffers, n));
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_step(uintptr_t opt, const uintptr_t *gradient_buffers, int n)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     Error e = H(opt)->opt->Step(pointers(gradient_buffers, n));
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
-uint64_t gmo_get_step_count(uintptr_t opt) {
-    if (!opt) { fail(Errorf("object handle is nil")); return 0; } return H(opt)->opt->GetStepCount(); }
-void gmo_update_learning_rate(uintptr_t opt, float lr) {
-    if (!opt) return; H(opt)->opt->UpdateLearningRate(lr); }
-void gmo_set_command_pool(uintptr_t opt, uintptr_t pool) {
-    if (!opt) return; H(opt)->opt->SetCommandPool(reinterpret_cast<Pointer>(pool)); }
-void gmo_cleanup(uintptr_t opt) {
-    if (!opt) return; H(opt)->opt->Cleanup(); }
+uint64_t gmo_get_step_count(uintptr_t opt)
+try {
+    if (!opt) {
+        fail(Errorf("object handle is nil"));
+        return 0;
+    }
+    return H(opt)->opt->GetStepCount();
+} catch (...) {
+    note_exception();
+    return 0;
+}
+
+void gmo_update_learning_rate(uintptr_t opt, float lr)
+try {
+    if (!opt) return;
+    H(opt)->opt->UpdateLearningRate(lr);
+} catch (...) {
+    note_exception();
+}
+
+void gmo_set_command_pool(uintptr_t opt, uintptr_t pool)
+try {
+    if (!opt) return;
+    H(opt)->opt->SetCommandPool(reinterpret_cast<Pointer>(pool));
+} catch (...) {
+    note_exception();
+}
+
+void gmo_cleanup(uintptr_t opt)
+try {
+    if (!opt) return;
+    H(opt)->opt->Cleanup();
+} catch (...) {
+    note_exception();
+}
+
 
 char *gmo_get_state_json(uintptr_t opt)
-{
+try {
     if (!opt) { fail(Errorf("object handle is nil")); return nullptr; }
     auto [state, err] = H(opt)->opt->GetState();
     if (!err.empty() || !state) {
@@ -225,19 +299,25 @@ char *gmo_get_state_json(uintptr_t opt)
     char *out = (char *)std::malloc(js.size() + 1);
     if (out) std::memcpy(out, js.c_str(), js.size() + 1);
     return out;
+} catch (...) {
+    note_exception();
+    return nullptr;
 }
 
 int gmo_load_state_json(uintptr_t opt, const char *json)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     auto [state, perr] = OptimizerState::FromJSON(json ? json : "");
     if (!perr.empty()) return fail(perr);
     Error e = H(opt)->opt->LoadState(&state);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 char *gmo_get_checkpoint_json(uintptr_t opt)
-{
+try {
     if (!opt) { fail(Errorf("object handle is nil")); return nullptr; }
     auto [state, err] = H(opt)->opt->GetState();
     if (!err.empty() || !state) {
@@ -249,19 +329,25 @@ char *gmo_get_checkpoint_json(uintptr_t opt)
     char *out = (char *)std::malloc(js.size() + 1);
     if (out) std::memcpy(out, js.c_str(), js.size() + 1);
     return out;
+} catch (...) {
+    note_exception();
+    return nullptr;
 }
 
 int gmo_load_checkpoint_json(uintptr_t opt, const char *json)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     auto [state, perr] = OptimizerState::FromCheckpointJSON(json ? json : "");
     if (!perr.empty()) return fail(perr);
     Error e = H(opt)->opt->LoadState(&state);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 float gmo_get_field(uintptr_t opt, const char *name)
-{
+try {
     if (!opt) return std::nanf("");
     Handle *h = H(opt);
     const std::string n = name ? name : "";
@@ -319,10 +405,13 @@ float gmo_get_field(uintptr_t opt, const char *name)
     }
     }
     return std::nanf("");
+} catch (...) {
+    note_exception();
+    return NAN;
 }
 
 uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index)
-{
+try {
     if (!opt) { fail(Errorf("object handle is nil")); return 0; }
     Handle *h = H(opt);
     const std::string t = state_type ? state_type : "";
@@ -362,10 +451,13 @@ uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index)
     }
     if (!v || index < 0 || index >= (int)v->size()) return 0;
     return reinterpret_cast<uintptr_t>((*v)[index]);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 int gmo_uses_pooling(uintptr_t opt)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     Handle *h = H(opt);
     switch (h->kind) {
@@ -377,14 +469,19 @@ int gmo_uses_pooling(uintptr_t opt)
     case GMO_NADAM: return static_cast<NadamOptimizerState *>(h->opt.get())->usePooling;
     }
     return 0;
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 void gmo_set_log_progress(uintptr_t opt, int on)
-{
+try {
     if (!opt) return;
     Handle *h = H(opt);
     if (h->kind == GMO_ADAGRAD) static_cast<AdaGradOptimizerState *>(h->opt.get())->logProgress = on != 0;
     if (h->kind == GMO_ADADELTA) static_cast<AdaDeltaOptimizerState *>(h->opt.get())->logProgress = on != 0;
+} catch (...) {
+    note_exception();
 }
 
 static AdamOptimizerState *adam_of(uintptr_t opt)
@@ -396,17 +493,20 @@ static AdamOptimizerState *adam_of(uintptr_t opt)
 
 int gmo_enable_mixed_precision(uintptr_t opt, float initial_scale, float growth_factor, float backoff_factor,
                                int growth_interval)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     auto *a = adam_of(opt);
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
     Error e = a->EnableMixedPrecision(initial_scale, growth_factor, backoff_factor, growth_interval);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_step_amp(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n,
                  int *skipped)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     auto *a = adam_of(opt);
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
@@ -414,36 +514,51 @@ int gmo_step_amp(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintp
     if (!e.empty()) return fail(e);
     if (skipped) *skipped = sk ? 1 : 0;
     return ok();
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_step_amp_async(uintptr_t opt, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n)
-{
+try {
     auto *a = adam_of(opt);
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
     Error e = a->StepAMPAsync(pointers(gradient16_buffers, n), pointers(weight16_buffers, weight16_buffers ? n : 0));
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_sync_amp(uintptr_t opt, uint64_t *skipped_steps)
-{
+try {
     auto *a = adam_of(opt);
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
     Error e = a->SyncAMP(skipped_steps);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 float gmo_loss_scale(uintptr_t opt)
-{
+try {
     if (!opt) return std::nanf("");
     auto *a = adam_of(opt);
     return a ? a->LossScale : std::nanf("");
+} catch (...) {
+    note_exception();
+    return NAN;
 }
 
 int gmo_growth_tracker(uintptr_t opt)
-{
+try {
     if (!opt) return fail(Errorf("object handle is nil"));
     auto *a = adam_of(opt);
     return a ? a->GrowthTracker : -1;
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 // ---- optimizer/lbfgs.go ----
@@ -451,7 +566,7 @@ static LBFGSOptimizerState *L(uintptr_t h) { return reinterpret_cast<LBFGSOptimi
 
 void gmo_lbfgs_default_config(int *history_size, float *line_search_tol, int *max_line_search, float *c1,
                               float *c2, float *initial_step)
-{
+try {
     const LBFGSConfig d = DefaultLBFGSConfig();
     if (history_size) *history_size = d.HistorySize;
     if (line_search_tol) *line_search_tol = d.LineSearchTol;
@@ -459,12 +574,14 @@ void gmo_lbfgs_default_config(int *history_size, float *line_search_tol, int *ma
     if (c1) *c1 = d.C1;
     if (c2) *c2 = d.C2;
     if (initial_step) *initial_step = d.InitialStep;
+} catch (...) {
+    note_exception();
 }
 
 uintptr_t gmo_lbfgs_new(int history_size, float line_search_tol, int max_line_search, float c1, float c2,
                         float initial_step, const int *dims, const int *ndims, int num_weights,
                         uintptr_t memory_manager, uintptr_t device)
-{
+try {
     Shapes shapes;
     const int *d = dims;
     for (int k = 0; k < num_weights; k++) {
@@ -480,75 +597,125 @@ uintptr_t gmo_lbfgs_new(int history_size, float line_search_tol, int max_line_se
     }
     ok();
     return reinterpret_cast<uintptr_t>(opt.release());
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void gmo_lbfgs_free(uintptr_t lbfgs) { delete L(lbfgs); }
 
 int gmo_lbfgs_set_weight_buffers(uintptr_t lbfgs, const uintptr_t *buffers, int n)
-{
+try {
     if (!lbfgs) return fail(Errorf("object handle is nil"));
     Error e = L(lbfgs)->SetWeightBuffers(pointers(buffers, n));
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_lbfgs_step(uintptr_t lbfgs, const uintptr_t *gradient_buffers, int n, float current_loss)
-{
+try {
     if (!lbfgs) return fail(Errorf("object handle is nil"));
     Error e = L(lbfgs)->Step(pointers(gradient_buffers, n), current_loss);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 void gmo_lbfgs_set_command_pool(uintptr_t lbfgs, uintptr_t pool)
-{
+try {
     if (!lbfgs) return;
     L(lbfgs)->SetCommandPool(reinterpret_cast<Pointer>(pool));
+} catch (...) {
+    note_exception();
 }
 
-int gmo_lbfgs_uses_pooling(uintptr_t lbfgs) {
-    if (!lbfgs) return fail(Errorf("object handle is nil")); return L(lbfgs)->usePooling ? 1 : 0; }
-uint64_t gmo_lbfgs_get_step(uintptr_t lbfgs) {
-    if (!lbfgs) { fail(Errorf("object handle is nil")); return 0; } return L(lbfgs)->GetStep(); }
+int gmo_lbfgs_uses_pooling(uintptr_t lbfgs)
+try {
+    if (!lbfgs) return fail(Errorf("object handle is nil"));
+    return L(lbfgs)->usePooling ? 1 : 0;
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+uint64_t gmo_lbfgs_get_step(uintptr_t lbfgs)
+try {
+    if (!lbfgs) {
+        fail(Errorf("object handle is nil"));
+        return 0;
+    }
+    return L(lbfgs)->GetStep();
+} catch (...) {
+    note_exception();
+    return 0;
+}
+
 
 void gmo_lbfgs_get_stats(uintptr_t lbfgs, uint64_t *step, int *history_size, int *history_used, float *prev_loss)
-{
+try {
     if (!lbfgs) return;
     auto stats = L(lbfgs)->GetStats();
     if (step) *step = std::get<uint64_t>(stats.at("step"));
     if (history_size) *history_size = (int)std::get<uint64_t>(stats.at("history_size"));
     if (history_used) *history_used = (int)std::get<uint64_t>(stats.at("history_used"));
     if (prev_loss) *prev_loss = std::get<float>(stats.at("prev_loss"));
+} catch (...) {
+    note_exception();
 }
 
 void gmo_lbfgs_history(uintptr_t lbfgs, int *count, int *index, float *last_step_size)
-{
+try {
     if (!lbfgs) return;
     if (count) *count = L(lbfgs)->historyCount;
     if (index) *index = L(lbfgs)->historyIndex;
     if (last_step_size) *last_step_size = L(lbfgs)->lastStepSize;
+} catch (...) {
+    note_exception();
 }
 
-void gmo_lbfgs_cleanup(uintptr_t lbfgs) {
-    if (!lbfgs) return; L(lbfgs)->Cleanup(); }
+void gmo_lbfgs_cleanup(uintptr_t lbfgs)
+try {
+    if (!lbfgs) return;
+    L(lbfgs)->Cleanup();
+} catch (...) {
+    note_exception();
+}
+
 
 int gmo_lbfgs_update_learning_rate(uintptr_t lbfgs, float lr)
-{
+try {
     if (!lbfgs) return fail(Errorf("object handle is nil"));
     Error e = L(lbfgs)->UpdateLearningRate(lr);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
-void gmo_lbfgs_set_log_progress(uintptr_t lbfgs, int on) {
-    if (!lbfgs) return; L(lbfgs)->logProgress = on != 0; }
+void gmo_lbfgs_set_log_progress(uintptr_t lbfgs, int on)
+try {
+    if (!lbfgs) return;
+    L(lbfgs)->logProgress = on != 0;
+} catch (...) {
+    note_exception();
+}
+
 
 int gmo_lbfgs_buffer_size(uintptr_t lbfgs, int index)
-{
+try {
     if (!lbfgs) return fail(Errorf("object handle is nil"));
     auto *l = L(lbfgs);
     return index >= 0 && (size_t)index < l->bufferSizes.size() ? l->bufferSizes[index] : -1;
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 uintptr_t gmo_lbfgs_buffer(uintptr_t lbfgs, const char *which, int history, int index)
-{
+try {
     if (!lbfgs) { fail(Errorf("object handle is nil")); return 0; }
     auto *l = L(lbfgs);
     const std::string w = which ? which : "";
@@ -563,12 +730,15 @@ uintptr_t gmo_lbfgs_buffer(uintptr_t lbfgs, const char *which, int history, int 
     else if (w == "search_dir" && i_ok) p = l->searchDir[index];
     else if (w == "weight" && i_ok) p = l->WeightBuffers[index];
     return reinterpret_cast<uintptr_t>(p);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 static memory::Tensor *T(uintptr_t h) { return reinterpret_cast<memory::Tensor *>(h); }
 
 uintptr_t gmo_tensor_new(const int *shape, int ndims, int dtype, int device_type)
-{
+try {
     auto [t, err] = memory::Tensor::NewTensor(std::vector<int>(shape, shape + (ndims > 0 ? ndims : 0)),
                                               (memory::DataType)dtype, (memory::DeviceType)device_type);
     if (!err.empty()) {
@@ -577,24 +747,73 @@ uintptr_t gmo_tensor_new(const int *shape, int ndims, int dtype, int device_type
     }
     ok();
     return reinterpret_cast<uintptr_t>(t);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
-uintptr_t gmo_tensor_retain(uintptr_t tensor) {
-    if (!tensor) { fail(Errorf("object handle is nil")); return 0; } return reinterpret_cast<uintptr_t>(T(tensor)->Retain()); }
-void gmo_tensor_release(uintptr_t tensor) {
-    if (!tensor) return; if (tensor) T(tensor)->Release(); }
+uintptr_t gmo_tensor_retain(uintptr_t tensor)
+try {
+    if (!tensor) {
+        fail(Errorf("object handle is nil"));
+        return 0;
+    }
+    return reinterpret_cast<uintptr_t>(T(tensor)->Retain());
+} catch (...) {
+    note_exception();
+    return 0;
+}
+
+void gmo_tensor_release(uintptr_t tensor)
+try {
+    if (tensor) T(tensor)->Release();
+} catch (...) {
+    note_exception();
+}
+
 void gmo_tensor_free(uintptr_t tensor) { delete T(tensor); }
-uintptr_t gmo_tensor_buffer(uintptr_t tensor) {
-    if (!tensor) { fail(Errorf("object handle is nil")); return 0; } return reinterpret_cast<uintptr_t>(T(tensor)->MetalBuffer()); }
-int gmo_tensor_size(uintptr_t tensor) {
-    if (!tensor) return fail(Errorf("object handle is nil")); return T(tensor)->Size(); }
-int gmo_tensor_ref_count(uintptr_t tensor) {
-    if (!tensor) return fail(Errorf("object handle is nil")); return T(tensor)->RefCount(); }
-int gmo_tensor_dtype(uintptr_t tensor) {
-    if (!tensor) return fail(Errorf("object handle is nil")); return (int)T(tensor)->DType(); }
+uintptr_t gmo_tensor_buffer(uintptr_t tensor)
+try {
+    if (!tensor) {
+        fail(Errorf("object handle is nil"));
+        return 0;
+    }
+    return reinterpret_cast<uintptr_t>(T(tensor)->MetalBuffer());
+} catch (...) {
+    note_exception();
+    return 0;
+}
+
+int gmo_tensor_size(uintptr_t tensor)
+try {
+    if (!tensor) return fail(Errorf("object handle is nil"));
+    return T(tensor)->Size();
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+int gmo_tensor_ref_count(uintptr_t tensor)
+try {
+    if (!tensor) return fail(Errorf("object handle is nil"));
+    return T(tensor)->RefCount();
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+int gmo_tensor_dtype(uintptr_t tensor)
+try {
+    if (!tensor) return fail(Errorf("object handle is nil"));
+    return (int)T(tensor)->DType();
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
 
 uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype)
-{
+try {
     if (!tensor) { fail(Errorf("object handle is nil")); return 0; }
     auto [t, err] = T(tensor)->ConvertTo((memory::DataType)dtype);
     if (!err.empty()) {
@@ -603,17 +822,23 @@ uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype)
     }
     ok();
     return reinterpret_cast<uintptr_t>(t);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 int gmo_tensor_copy_float32_data(uintptr_t tensor, const float *data, int n)
-{
+try {
     if (!tensor) return fail(Errorf("object handle is nil"));
     Error e = T(tensor)->CopyFloat32Data(std::vector<float>(data, data + (n > 0 ? n : 0)));
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity)
-{
+try {
     if (!tensor) return fail(Errorf("object handle is nil"));
     auto [data, err] = T(tensor)->ToFloat32Slice();
     if (!err.empty()) return fail(err);
@@ -621,23 +846,32 @@ int gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity)
     std::memcpy(out, data.data(), data.size() * sizeof(float));
     ok();
     return (int)data.size();
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_tensor_copy_from(uintptr_t dst, uintptr_t src)
-{
+try {
     if (!dst) return fail(Errorf("object handle is nil"));
     Error e = T(dst)->CopyFrom(T(src));
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_calculate_size(const int *shape, int ndims, int dtype)
-{
+try {
     return memory::calculateSize(std::vector<int>(shape, shape + (ndims > 0 ? ndims : 0)), (memory::DataType)dtype);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *weight_tensors, int num_weights,
                                                 const uintptr_t *gradient_tensors, int num_gradients)
-{
+try {
     std::vector<memory::Tensor *> w, g;     // a nil optimizer is the engine's own error case
     for (int k = 0; k < num_weights; k++) w.push_back(T(weight_tensors[k]));
     for (int k = 0; k < num_gradients; k++) g.push_back(T(gradient_tensors[k]));
@@ -645,6 +879,9 @@ int gmo_execute_step_with_precomputed_gradients(uintptr_t opt, const uintptr_t *
     Handle *h = H(opt);
     Error e = engine::ExecuteStepWithPrecomputedGradients(h ? h->opt.get() : nullptr, w, g, h ? names[h->kind] : "Adam");
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 struct SchedulerHandle {
@@ -654,7 +891,7 @@ struct SchedulerHandle {
 };
 
 uintptr_t gmo_scheduler_new(int kind, int a, double b, double c, const char *mode)
-{
+try {
     auto *h = new SchedulerHandle{kind, nullptr, ""};
     switch (kind) {
     case 0: h->s = std::make_unique<training::StepLRScheduler>(a, b); break;
@@ -666,33 +903,55 @@ uintptr_t gmo_scheduler_new(int kind, int a, double b, double c, const char *mod
     }
     h->name = h->s->GetName();
     return reinterpret_cast<uintptr_t>(h);
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 void gmo_scheduler_free(uintptr_t scheduler) { delete reinterpret_cast<SchedulerHandle *>(scheduler); }
 
 double gmo_scheduler_get_lr(uintptr_t scheduler, int epoch, int step, double base_lr)
-{
+try {
     if (!scheduler) return std::nan("");
     return reinterpret_cast<SchedulerHandle *>(scheduler)->s->GetLR(epoch, step, base_lr);
+} catch (...) {
+    note_exception();
+    return NAN;
 }
 
 double gmo_scheduler_plateau_step(uintptr_t scheduler, double metric, double current_lr)
-{
+try {
     if (!scheduler) return std::nan("");
     auto *h = reinterpret_cast<SchedulerHandle *>(scheduler);
     if (h->kind != 3) return std::nan("");
     return static_cast<training::ReduceLROnPlateauScheduler *>(h->s.get())->Step(metric, current_lr);
+} catch (...) {
+    note_exception();
+    return NAN;
 }
 
-const char *gmo_scheduler_name(uintptr_t scheduler) {
-    if (!scheduler) { fail(Errorf("object handle is nil")); return ""; } return reinterpret_cast<SchedulerHandle *>(scheduler)->name.c_str(); }
+const char *gmo_scheduler_name(uintptr_t scheduler)
+try {
+    if (!scheduler) {
+        fail(Errorf("object handle is nil"));
+        return "";
+    }
+    return reinterpret_cast<SchedulerHandle *>(scheduler)->name.c_str();
+} catch (...) {
+    note_exception();
+    return nullptr;
+}
+
 
 double gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, int step, double base_lr)
-{
+try {
     if (!scheduler) return std::nan("");
     const double lr = gmo_scheduler_get_lr(scheduler, epoch, step, base_lr);
     if (opt) H(opt)->opt->UpdateLearningRate((float)lr);
     return lr;
+} catch (...) {
+    note_exception();
+    return NAN;
 }
 
 float gmo_pow(float x, float y) { return optimizer::pow(x, y); }
@@ -700,8 +959,11 @@ float gmo_pow(float x, float y) { return optimizer::pow(x, y); }
 int gmo_extract_buffer_index(const char *name) { return extractBufferIndex(name ? name : ""); }
 
 int gmo_calculate_tensor_size(const int *dims, int ndims)
-{
+try {
     return calculateTensorSize(std::vector<int>(dims, dims + (ndims > 0 ? ndims : 0)));
+} catch (...) {
+    note_exception();
+    return -1;
 }
 
 }  // extern "C"

@@ -96,6 +96,11 @@ int copy_buffer_to_buffer_sync(uintptr_t src_buffer, uintptr_t dst_buffer, int s
 /* -3 no usable GPU stream; others per function.  A tensor whose allocation   */
 /* (when the handle is one of this library's) is shorter than buffer_sizes[i] */
 /* is skipped, as the reference does (bridge_optimizer.m:427-436).            */
+/* No C++ exception crosses this boundary: one caught inside an entry point   */
+/* (a failed host allocation, say) returns the code the reference returns     */
+/* from its own @catch block: the "HIP error" code of each function below     */
+/* (-13 for execute_adam_step_mpsgraph_pooled, .m:683-686), with the reason   */
+/* in gm_last_error().                                                        */
 /* ------------------------------------------------------------------------ */
 
 /* bridge_optimizer.h:11-23 / .m:160-357.  momentum_buffers may be NULL or hold

@@ -339,3 +339,21 @@ def test_nil_object_handles_are_errors_not_crashes():
                                           (-2.0, 2.0, 4.0), (1.5, 2.0, 2.25)])
 def test_pow_helper(x, y, expected):                        # adam_test.go:282-308
     assert lib.gmo_pow(x, y) == expected
+
+
+def test_a_cpp_exception_stops_at_the_c_boundary(mm):
+    """A standard-library exception inside an entry point (here: a negative dimension count, which makes the
+    shape vector's constructor throw std::length_error) must come back as the entry point's failure value with
+    the reason in gmo_last_error(), not unwind into the caller's C, Go or Python frames."""
+    import ctypes
+    cfg = (ctypes.c_float * 6)(0.01, 0, 0, 0, 0, 0)
+    dims = (ctypes.c_int * 1)(4)
+    ndims = (ctypes.c_int * 1)(-1)
+    h = lib.gmo_optimizer_new(pkg.KINDS["sgd"], cfg, dims, ndims, 1, mm, MOCK_DEVICE)
+    assert h == 0
+    assert lib.gmo_last_error().decode().startswith("exception: ")
+    # the library is still usable afterwards
+    ndims[0] = 1
+    h = lib.gmo_optimizer_new(pkg.KINDS["sgd"], cfg, dims, ndims, 1, mm, MOCK_DEVICE)
+    assert h != 0
+    lib.gmo_optimizer_free(h)
