@@ -36,7 +36,7 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
 # file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
 MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10,
                         # bytes per step, summed over the passes of a 10-pair step (profiles/lbfgs_c5_1b_hbm_traffic.md)
-                        ("lbfgs-c5", 10): 360.72 * 1012301824}
+                        ("lbfgs-c5", 10): 352.68 * 1012301824}
 
 from workloads import amp_125m_sizes, cnn_sizes, ragged_sizes, transformer_block_sizes  # noqa: E402
 
@@ -131,14 +131,14 @@ LBFGS_WORKLOADS = {
 
 
 def lbfgs_bytes_per_param(valid_pairs):
-    """Algorithmic HBM bytes per parameter of one L-BFGS step with a non-empty history of two or more
-    slots: every pass reads its operands once and writes its result once.  The last pass is the update
-    with the curvature pass riding on it: it reads r (or nothing, when no pair is valid: r = -g), w, g,
-    s_prev and writes p, w, old_g, s_cur, y_prev.  No valid pair: 12 + 20 = 32.  c valid pairs: init (12)
-    + c backward (16; the last one 12, its dot operand y_0 being the buffer its axpy reads) + c forward
-    (16; the last one 12, no dot) + update with curvature (16 + 20)."""
+    """Algorithmic HBM bytes per parameter of one L-BFGS step with a non-empty history: every pass reads its
+    operands once and writes its result once.  The last pass is the update: it reads r (or nothing, when no
+    pair is valid: r = -g is formed from the gradient it reads anyway), w, g and writes p, w, old_g, s_cur,
+    y_prev.  No valid pair: 8 + 20 = 28.  c valid pairs: first dot product (8: q = -g is not stored) + c
+    backward (16; the last one 12, its dot operand y_0 being the buffer its axpy reads) + c forward (16; the last
+    one 12, no dot) + update (12 + 20)."""
     c = valid_pairs
-    return 32 if c == 0 else 12 + (16 * c - 4) + (16 * c - 4) + 36
+    return 28 if c == 0 else 8 + (16 * c - 4) + (16 * c - 4) + 32
 
 
 def bench_lbfgs(args, pkg, dev):

@@ -8,16 +8,23 @@
 // so a history pair costs two passes, not four:
 //
 //   prologue     gather rho[idx(j)], mark pairs with |rho| < 1e-10 invalid, alpha[j] = 0 for them
-//   init         q = -g                       (+ dot(s_j, q) for the newest valid pair)
-//   backward     q -= alpha_j y_j             (+ dot with the next operand)
+//   init         dot(s_j, q), q = -g, for the newest valid pair (q stays in registers)
+//   backward     q -= alpha_j y_j             (+ dot with the next operand; the first one reads g for q)
 //   forward      r += (alpha_j - beta) s_j    (+ dot with the next operand)
-//   update       p = -r; x += a p; old_g = g; s_cur = a p
-//   curvature    y_prev = g - old_g; rho_prev from dot(s_prev, y_prev)
+//   update       p = -r; x += a p; old_g = g; s_cur = a p; y_prev = g - old_g; rho_prev = 0
+//
+// The last line is the reference's curvature update as its own order of statements makes it
+// come out.  It copies g into old_g (bridge_optimizer.m:1236-1239) before it forms
+// y_prev = g - old_g (:1285-1288), so every element of y_prev is g - g: +0, or NaN for a
+// non-finite g.  s_prev . y_prev is then a sum of zeros and NaNs, |s.y| > 1e-10 is false either
+// way, and rho_prev = 0 (:1302-1308), whatever s_prev holds.  The update pass therefore writes
+// y_prev = g - g from the gradient it already holds and rho_prev is set to 0 without reading
+// s_prev or summing anything: the same bits as the reference's loop nest, 8 bytes per element
+// less traffic.
 //
 // Which pairs are valid is read back once per step (history_count flags), so
 // only the passes that do work are launched; with the history the reference's
-// own optimizer produces (every rho it writes is 0) a step is the update pass
-// and the curvature pass.
+// own optimizer produces (every rho it writes is 0) a step is the update pass alone.
 //
 // Dot products: exact fp64 products, summed in fp64 by a fixed radix-1024 tree
 // (lane l of a 256-lane workgroup adds elements l, l+256, l+512, l+768 of a
@@ -164,29 +171,25 @@ __device__ inline double workgroup_tree(double v)
     return (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
 }
 
-enum : int { kModeInit = 0, kModeAxpy, kModeUpdate, kModeUpdateFromGrad, kModeCurvature, kModeDotOnly };
+enum : int { kModeAxpy = 0, kModeAxpyFirst };
 
 struct StreamArgs {
     const LbChunk *chunks;
     uint32_t slice_shift;
     // rows of the handle table (one device address per tensor); meaning depends on the mode
-    const uintptr_t *r0, *r1, *r2, *r3, *r4, *r5, *r6;
+    const uintptr_t *r0, *r1, *r2, *r3;
     double *partial;               // slice sums (modes with a dot product)
     const LbScalars *scalars;      // coefficient for kModeAxpy
-    float step;                    // kModeUpdate*
     int subtract;                  // kModeAxpy: x - c v (backward loop) or x + c v (forward loop)
 };
 
 // One workgroup = one 1024-element slice: lane l handles elements l, l+256, l+512, l+768.
-//   kModeInit            r0 = g, r1 = direction, r2 = dot operand        q = -g
+//   kModeAxpyFirst       r0 = g, r1 = v, r2 = dot operand, r3 = direction    x = (-g) - c v, stored as the direction
 //   kModeAxpy            r0 = direction, r1 = v, r2 = dot operand        x = x -/+ c v
-//   kModeUpdate          r0 = direction, r1 = w, r2 = g, r3 = old_g, r4 = s_cur
-//   kModeUpdateFromGrad  same, with r = -g formed in registers (no valid pair this step)
-//                        with DOT, both update modes also run the curvature pass on the values
-//                        they hold: r5 = s_prev, r6 = y_prev; y = g - g', g' being the gradient
-//                        just stored as old_g, and dot(s_prev, y)
-//   kModeCurvature       r0 = g, r1 = old_g, r2 = s_prev, r3 = y_prev    y = g - old_g, dot(s, y)
-//   kModeDotOnly         r0 = a, r1 = b
+// The recursion starts from q = -g.  Nothing but its first axpy reads that q, so it is formed in
+// registers twice (for the first dot product, lbfgs_dot_kernel, and by the first axpy, which reads
+// g instead of the direction buffer) rather than written out and read back: 4 bytes per element
+// less.
 template <int MODE, bool DOT, bool NT>
 __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
 {
@@ -199,43 +202,28 @@ __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
 
     float *p0 = reinterpret_cast<float *>(a.r0[ch.tensor]) + first;
     float *p1 = reinterpret_cast<float *>(a.r1[ch.tensor]) + first;
-    float *p2 = nullptr, *p3 = nullptr, *p4 = nullptr;
-    constexpr bool kFusedDot = DOT && (MODE == kModeInit || MODE == kModeAxpy);   // r2 = dot operand
-    if (kFusedDot || MODE == kModeUpdate || MODE == kModeUpdateFromGrad || MODE == kModeCurvature)
-        p2 = reinterpret_cast<float *>(a.r2[ch.tensor]) + first;
-    if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad || MODE == kModeCurvature)
-        p3 = reinterpret_cast<float *>(a.r3[ch.tensor]) + first;
-    if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad)
-        p4 = reinterpret_cast<float *>(a.r4[ch.tensor]) + first;
-    constexpr bool kFusedCurvature = DOT && (MODE == kModeUpdate || MODE == kModeUpdateFromGrad);
-    float *p5 = nullptr, *p6 = nullptr;
-    if (kFusedCurvature) {
-        p5 = reinterpret_cast<float *>(a.r5[ch.tensor]) + first;
-        p6 = reinterpret_cast<float *>(a.r6[ch.tensor]) + first;
-    }
+    float *p2 = nullptr;
+    constexpr bool kFusedDot = DOT;                                           // r2 = dot operand
+    if (kFusedDot) p2 = reinterpret_cast<float *>(a.r2[ch.tensor]) + first;
+    float *out = p0;                                                          // where an axpy stores x
+    if (MODE == kModeAxpyFirst) out = reinterpret_cast<float *>(a.r3[ch.tensor]) + first;
 
-    float coef = 0.0f;
-    if (MODE == kModeAxpy) coef = a.scalars->coef;
+    const float coef = a.scalars->coef;
 
     // Order of a lane's memory operations: element by element, all loads of the element, then
-    // its stores.  The compiler cannot prove that the streams do not overlap, so a store orders
+    // its store.  The compiler cannot prove that the streams do not overlap, so a store orders
     // the loads around it; a store placed between two loads of one element leaves a single load
-    // in flight per lane (the init pass ran at 53 % of peak that way, 75 % with loads first).
+    // in flight per lane (a pass ran at 53 % of peak that way, 75 % with loads first).
     // Hoisting the loads of all four elements above the first store is slower for the passes
     // that feed a dot product (68 % against 86 % of peak): reads and writes then reach the
     // memory controllers in bursts instead of finely interleaved.
-    constexpr bool kLoad0 = MODE != kModeUpdateFromGrad;
-    constexpr bool kLoad1 = MODE != kModeInit;
-    constexpr bool kLoad2 = kFusedDot || MODE == kModeUpdate || MODE == kModeUpdateFromGrad ||
-                            MODE == kModeCurvature;
-    float v0[kPerLane], v1[kPerLane], v2[kPerLane], v3[kPerLane];
+    float v0[kPerLane], v1[kPerLane], v2[kPerLane];
     auto load_element = [&](int u) {
         const size_t o = (size_t)u * kLanes;
         const bool ok = threadIdx.x + u * kLanes < left;
-        v0[u] = (kLoad0 && ok) ? ld<NT>(p0 + o) : 0.0f;
-        v1[u] = (kLoad1 && ok) ? ld<NT>(p1 + o) : 0.0f;
-        v2[u] = (kLoad2 && ok) ? ld<NT>(p2 + o) : 0.0f;
-        v3[u] = (kFusedCurvature && ok) ? ld<NT>(p5 + o) : 0.0f;
+        v0[u] = ok ? ld<NT>(p0 + o) : 0.0f;
+        v1[u] = ok ? ld<NT>(p1 + o) : 0.0f;
+        v2[u] = (kFusedDot && ok) ? ld<NT>(p2 + o) : 0.0f;
     };
     // arithmetic, stores, and the lane's running fp64 sum in element order
     double acc = 0.0;
@@ -244,44 +232,104 @@ __global__ void __launch_bounds__(kLanes) lbfgs_stream_kernel(StreamArgs a)
         load_element(u);
         if (threadIdx.x + u * kLanes >= left) continue;
         const size_t o = (size_t)u * kLanes;
-        float x = 0.0f, d = 0.0f;
-        if (MODE == kModeInit) {
-            x = -v0[u];
-            d = v2[u];
-            st<NT>(x, p1 + o);
-        } else if (MODE == kModeAxpy) {
-            const float cv = coef * v1[u];
-            x = a.subtract ? v0[u] - cv : v0[u] + cv;
-            d = v2[u];
-            st<NT>(x, p0 + o);
-        } else if (MODE == kModeUpdate || MODE == kModeUpdateFromGrad) {
-            const float g = v2[u];
-            const float r = MODE == kModeUpdate ? v0[u] : -g;
-            const float p = -r;
-            const float sp = a.step * p;
-            st<NT>(p, p0 + o);
-            st<NT>(v1[u] + sp, p1 + o);
-            st<NT>(g, p3 + o);
-            st<NT>(sp, p4 + o);
-            if (kFusedCurvature) {
-                x = g - g;          // y = g - old_g with old_g = g as just stored: +0, or NaN for a non-finite g
-                d = v3[u];
-                st<NT>(x, p6 + o);
-            }
-        } else if (MODE == kModeCurvature) {
-            x = v0[u] - v1[u];
-            d = v2[u];
-            st<NT>(x, p3 + o);
-        } else {   // kModeDotOnly
-            x = v0[u];
-            d = v1[u];
-        }
+        const float from = MODE == kModeAxpyFirst ? -v0[u] : v0[u];
+        const float cv = coef * v1[u];
+        const float x = a.subtract ? from - cv : from + cv;
+        const float d = v2[u];
+        st<NT>(x, out + o);
         if (DOT) acc = acc + (double)d * (double)x;     // exact product, one fp64 rounding per addition
     }
     if (DOT) {
         const double total = workgroup_tree(acc);
         if (threadIdx.x == 0) a.partial[ch.first_slice + slice] = total;
     }
+}
+
+// The passes that only read (dot(s, -g) at the head of the recursion, gm_lbfgs_dot): the same sum
+// as lbfgs_stream_kernel forms, with the memory side reshaped.  Nothing is stored, so what limits
+// a pure read is the bytes each wave keeps in flight: lane l loads elements 4 l .. 4 l + 3 of the
+// slice with one 16-byte load per operand, the four exact fp64 products go to LDS at their element
+// positions, and after a barrier lane l adds products l, l + 256, l + 512, l + 768 in that order:
+// the lane sum of the tree.  Slices that are ragged or not 16-byte aligned take 4-byte loads in
+// the tree's own lane order.  Measured on MI355X over 1B parameters: 8 B/param in 1.61 ms (63 % of
+// peak) with 4-byte loads throughout.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <bool NEGATE, bool NT>
+__global__ void __launch_bounds__(kLanes) lbfgs_dot_kernel(StreamArgs a)
+{
+    __shared__ double product[kSlice];
+    const LbChunk ch = a.chunks[blockIdx.x >> a.slice_shift];
+    const uint32_t slice = blockIdx.x & ((1u << a.slice_shift) - 1u);
+    const uint32_t base = slice * kSlice;
+    if (base >= ch.count) return;
+    const uint32_t left = ch.count - base;
+    const float *pa = reinterpret_cast<const float *>(a.r0[ch.tensor]) + ch.offset + base;
+    const float *pb = reinterpret_cast<const float *>(a.r1[ch.tensor]) + ch.offset + base;
+    double acc = 0.0;
+    const bool wide = left >= (uint32_t)kSlice &&
+                      ((reinterpret_cast<uintptr_t>(pa) | reinterpret_cast<uintptr_t>(pb)) & 15u) == 0;
+    if (wide) {                                        // uniform over the workgroup
+        const GM_GLOBAL floatx4 *ga = (const GM_GLOBAL floatx4 *)pa + threadIdx.x;
+        const GM_GLOBAL floatx4 *gb = (const GM_GLOBAL floatx4 *)pb + threadIdx.x;
+        const floatx4 x = NT ? __builtin_nontemporal_load(ga) : *ga;
+        const floatx4 d = NT ? __builtin_nontemporal_load(gb) : *gb;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float xv = NEGATE ? -x[c] : x[c];
+            product[4 * threadIdx.x + c] = (double)d[c] * (double)xv;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kPerLane; u++) acc = acc + product[threadIdx.x + u * kLanes];
+    } else {
+#pragma unroll
+        for (int u = 0; u < kPerLane; u++) {
+            const uint32_t i = threadIdx.x + u * kLanes;
+            if (i >= left) continue;
+            const float x0 = ld<NT>(pa + i);
+            const float xv = NEGATE ? -x0 : x0;
+            acc = acc + (double)ld<NT>(pb + i) * (double)xv;
+        }
+    }
+    const double total = workgroup_tree(acc);
+    if (threadIdx.x == 0) a.partial[ch.first_slice + slice] = total;
+}
+
+// The update pass: p = -r; x += a p; old_g = g; s_cur = a p; and, when the history is not empty,
+// y_prev = g - old_g with old_g = g as just stored (+0, or NaN for a non-finite g).  It feeds no
+// dot product, so it is free of the 1024-element slices of the summation tree: one element per
+// lane, a workgroup per 256 elements.  Five of its seven or eight streams are written, and the
+// write-heavy mix is the one that suffers most from long-lived workgroups: measured on MI355X over
+// 2^29 elements, 81 % of peak HBM bandwidth in this shape against 70 % with four strided elements
+// per lane (the shape of the passes above), 73-74 % with 8-byte lanes and 68-71 % with 16-byte lanes.
+struct UpdateArgs {
+    const LbChunk *chunks;
+    uint32_t quarter_shift;        // log2(256-element workgroups per chunk)
+    const uintptr_t *dir, *w, *g, *old_g, *s_cur, *y_prev;
+    float step;
+};
+
+template <bool FROM_GRADIENT, bool WITH_Y, bool NT>
+__global__ void __launch_bounds__(kLanes) lbfgs_update_kernel(UpdateArgs a)
+{
+    const LbChunk ch = a.chunks[blockIdx.x >> a.quarter_shift];
+    const uint32_t local = (blockIdx.x & ((1u << a.quarter_shift) - 1u)) * kLanes + threadIdx.x;
+    if (local >= ch.count) return;
+    const size_t i = (size_t)ch.offset + local;
+    float *dir = reinterpret_cast<float *>(a.dir[ch.tensor]) + i;
+    float *w = reinterpret_cast<float *>(a.w[ch.tensor]) + i;
+    const float g = ld<NT>(reinterpret_cast<const float *>(a.g[ch.tensor]) + i);
+    const float x = ld<NT>(w);
+    // r = -g when no pair is valid this step (formed in registers), else what the recursion left
+    const float r = FROM_GRADIENT ? -g : ld<NT>(dir);
+    const float p = -r;
+    const float sp = a.step * p;
+    st<NT>(p, dir);
+    st<NT>(x + sp, w);
+    st<NT>(g, reinterpret_cast<float *>(a.old_g[ch.tensor]) + i);
+    st<NT>(sp, reinterpret_cast<float *>(a.s_cur[ch.tensor]) + i);
+    if (WITH_Y) st<NT>(g - g, reinterpret_cast<float *>(a.y_prev[ch.tensor]) + i);
 }
 
 __device__ inline void run_epilogue(const Epilogue &e, double total)
@@ -423,7 +471,7 @@ bool ensure_geometry(Context *ctx, Plan &p, const int *sizes, int n)
     }
     p.slice_shift = 0;
     while ((1u << p.slice_shift) < (uint32_t)(chunk / kSlice)) p.slice_shift++;
-    if (slice > 0xFFFFFFFFull || ((uint64_t)chunks.size() << p.slice_shift) > 0x7FFFFFFFull) {
+    if (slice > 0xFFFFFFFFull || ((uint64_t)chunks.size() << (p.slice_shift + 2)) > 0x7FFFFFFFull) {
         set_error("tensor list too large for one launch");
         return false;
     }
@@ -549,6 +597,23 @@ int stage_handles(Context *ctx, Plan &p, int n, int m, const uintptr_t *w, const
     return 0;
 }
 
+// dot(b, a) or dot(b, -a): a.r0 = a rows, a.r1 = b rows
+void launch_dot(Context *ctx, const Plan &p, StreamArgs a, bool negate)
+{
+    if (p.num_chunks == 0) return;
+    const uint32_t grid = p.num_chunks << p.slice_shift;
+    a.chunks = p.d_chunks;
+    a.slice_shift = p.slice_shift;
+    const bool nt = current_nontemporal();
+    if (negate) {
+        if (nt) lbfgs_dot_kernel<true, true><<<grid, kLanes, 0, ctx->stream>>>(a);
+        else lbfgs_dot_kernel<true, false><<<grid, kLanes, 0, ctx->stream>>>(a);
+    } else {
+        if (nt) lbfgs_dot_kernel<false, true><<<grid, kLanes, 0, ctx->stream>>>(a);
+        else lbfgs_dot_kernel<false, false><<<grid, kLanes, 0, ctx->stream>>>(a);
+    }
+}
+
 template <int MODE, bool DOT>
 void launch_stream(Context *ctx, const Plan &p, StreamArgs a)
 {
@@ -558,6 +623,24 @@ void launch_stream(Context *ctx, const Plan &p, StreamArgs a)
     a.slice_shift = p.slice_shift;
     if (current_nontemporal()) lbfgs_stream_kernel<MODE, DOT, true><<<grid, kLanes, 0, ctx->stream>>>(a);
     else lbfgs_stream_kernel<MODE, DOT, false><<<grid, kLanes, 0, ctx->stream>>>(a);
+}
+
+void launch_update(Context *ctx, const Plan &p, UpdateArgs a, bool from_gradient, bool with_y)
+{
+    if (p.num_chunks == 0) return;
+    a.chunks = p.d_chunks;
+    a.quarter_shift = p.slice_shift + 2;      // four 256-element workgroups to a 1024-element slice
+    const uint32_t grid = p.num_chunks << a.quarter_shift;
+    const bool nt = current_nontemporal();
+    hipStream_t st = ctx->stream;
+#define GM_LAUNCH_UPDATE(F, Y)                                                        \
+    do {                                                                              \
+        if (nt) lbfgs_update_kernel<F, Y, true><<<grid, kLanes, 0, st>>>(a);         \
+        else lbfgs_update_kernel<F, Y, false><<<grid, kLanes, 0, st>>>(a);           \
+    } while (0)
+    if (from_gradient) { if (with_y) GM_LAUNCH_UPDATE(true, true); else GM_LAUNCH_UPDATE(true, false); }
+    else { if (with_y) GM_LAUNCH_UPDATE(false, true); else GM_LAUNCH_UPDATE(false, false); }
+#undef GM_LAUNCH_UPDATE
 }
 
 // Upper tree levels over the slice sums in d_partial[0], then the scalar epilogue.
@@ -671,32 +754,16 @@ try {
     StreamArgs base{};
     base.partial = p.d_partial[0];
     base.scalars = p.d_scalars;
-    base.step = initial_step;
 
-    // The curvature pass (y_prev = g - old_g, s_prev . y_prev) reads old_g right after the update
-    // pass has stored g into it, so it can ride on the update pass with the values in registers,
-    // unless the ring has one slot (s_prev is then the s the update pass is writing).
     const int prev = (history_index - 1 + m) % m;
-    const bool fuse_curvature = history_count > 0 && prev != history_index;
-    auto with_curvature = [&](StreamArgs a) {
-        a.r5 = r.s(prev, n);
-        a.r6 = r.y(prev, n);
-        return a;
-    };
 
-    if (valid.empty()) {
-        // q = -g, no recursion, p = -q: one pass
-        StreamArgs a = base;
-        a.r0 = r.dir; a.r1 = r.w; a.r2 = r.g; a.r3 = r.old_g; a.r4 = r.s(history_index, n);
-        if (fuse_curvature) launch_stream<kModeUpdateFromGrad, true>(ctx, p, with_curvature(a));
-        else launch_stream<kModeUpdateFromGrad, false>(ctx, p, a);
-    } else {
+    if (!valid.empty()) {
         const int count = (int)valid.size();
-        // q = -g, with the first dot product of the backward loop
+        // q = -g (:1031-1043) stays in registers: the first dot product of the backward loop
         {
             StreamArgs a = base;
-            a.r0 = r.g; a.r1 = r.dir; a.r2 = r.s(slot(valid[count - 1]), n);
-            launch_stream<kModeInit, true>(ctx, p, a);
+            a.r0 = r.g; a.r1 = r.s(slot(valid[count - 1]), n);
+            launch_dot(ctx, p, a, true);
         }
         // backward loop, newest pair first (bridge_optimizer.m:1046-1137)
         for (int k = count - 1; k >= 0; k--) {
@@ -706,7 +773,13 @@ try {
             a.r0 = r.dir; a.r1 = r.y(idx, n); a.subtract = 1;
             // next dot: s of the next older valid pair, or y of the oldest one (first forward dot)
             a.r2 = k > 0 ? r.s(slot(valid[k - 1]), n) : r.y(slot(valid[0]), n);
-            launch_stream<kModeAxpy, true>(ctx, p, a);
+            if (k == count - 1) {
+                // the first axpy forms q = -g from the gradient and stores the result as the direction
+                a.r0 = r.g; a.r3 = r.dir;
+                launch_stream<kModeAxpyFirst, true>(ctx, p, a);
+            } else {
+                launch_stream<kModeAxpy, true>(ctx, p, a);
+            }
         }
         // forward loop, oldest pair first (:1143-1216)
         for (int k = 0; k < count; k++) {
@@ -721,23 +794,20 @@ try {
                 launch_stream<kModeAxpy, false>(ctx, p, a);
             }
         }
-        // p = -r; x += a p; old_g = g; s_cur = a p  (:1219-1276)
-        StreamArgs a = base;
-        a.r0 = r.dir; a.r1 = r.w; a.r2 = r.g; a.r3 = r.old_g; a.r4 = r.s(history_index, n);
-        if (fuse_curvature) launch_stream<kModeUpdate, true>(ctx, p, with_curvature(a));
-        else launch_stream<kModeUpdate, false>(ctx, p, a);
+    }
+    // p = -r (r = -g when no pair took part); x += a p; old_g = g; s_cur = a p  (:1219-1259), and with a
+    // non-empty history y_prev = g - old_g, rho_prev = 0  (:1262-1310)
+    {
+        UpdateArgs u{};
+        u.dir = r.dir; u.w = r.w; u.g = r.g; u.old_g = r.old_g; u.s_cur = r.s(history_index, n);
+        u.y_prev = r.y(prev, n);
+        u.step = initial_step;
+        launch_update(ctx, p, u, valid.empty(), history_count > 0);
     }
     if (step_size) *step_size = initial_step;
-
-    // y_prev = g - old_g, rho_prev = 1 / (s_prev . y_prev)  (:1279-1335)
-    if (history_count > 0) {
-        if (!fuse_curvature) {
-            StreamArgs a = base;
-            a.r0 = r.g; a.r1 = r.old_g; a.r2 = r.s(prev, n); a.r3 = r.y(prev, n);
-            launch_stream<kModeCurvature, true>(ctx, p, a);
-        }
-        launch_reduction(ctx, p, Epilogue{kOpRho, nullptr, nullptr, rho_ptr(prev), p.d_scalars});
-    }
+    if (history_count > 0)
+        lbfgs_epilogue_kernel<<<1, 64, 0, stream>>>(nullptr, 0, Epilogue{kOpRho, nullptr, nullptr, rho_ptr(prev),
+                                                                        p.d_scalars});
     return hip_ok(hipGetLastError(), "L-BFGS kernel launch") ? 0 : -8;
 } catch (...) {
     note_exception();
@@ -801,7 +871,7 @@ try {
         a.scalars = p.d_scalars;
         a.r0 = d_rows;
         a.r1 = d_rows + n;
-        launch_stream<kModeDotOnly, true>(ctx, p, a);
+        launch_dot(ctx, p, a, false);
         launch_reduction(ctx, p, Epilogue{kOpStore, nullptr, nullptr, nullptr, p.d_scalars});
         if (hip_ok(hipGetLastError(), "dot kernel launch") &&
             hip_ok(hipMemcpyAsync(h_result, p.d_scalars, sizeof(LbScalars), hipMemcpyDeviceToHost, ctx->stream),

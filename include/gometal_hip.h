@@ -187,7 +187,9 @@ int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
  * search: c1, c2, max_line_search and the losses are ignored, as in the reference);
  * old_g = g; s[history_index] = initial_step * p; and, when history_count > 0,
  * y[prev] = g - old_g and rho[prev] = 1 / (s[prev] . y[prev]) (0 when |s.y| <= 1e-10) for
- * prev = history_index - 1.  s_vectors_flat / y_vectors_flat hold history_size * num_weights
+ * prev = history_index - 1.  In that order old_g already equals g, so y[prev] is g - g
+ * (+0, NaN for a non-finite g) and rho[prev] is 0: that is what the reference's code yields
+ * and what this call writes, without summing s[prev] . y[prev].  s_vectors_flat / y_vectors_flat hold history_size * num_weights
  * handles, entry [h * num_weights + i]; rho_buffers holds history_size handles of 4-byte
  * buffers; alpha_buffer holds history_size floats.  *step_size = initial_step.
  * Dot products are exact fp64 products summed by a fixed tree and rounded once to fp32
