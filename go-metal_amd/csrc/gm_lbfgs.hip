@@ -17,7 +17,7 @@
 // come out.  It copies g into old_g (bridge_optimizer.m:1236-1239) before it forms
 // y_prev = g - old_g (:1285-1288), so every element of y_prev is g - g: +0, or NaN for a
 // non-finite g.  s_prev . y_prev is then a sum of zeros and NaNs, |s.y| > 1e-10 is false either
-// way, and rho_prev = 0 (:1302-1308), whatever s_prev holds.  The update pass therefore writes
+// way, and rho_prev = 0 (:1304-1310), whatever s_prev holds.  The update pass therefore writes
 // y_prev = g - g from the gradient it already holds and rho_prev is set to 0 without reading
 // s_prev or summing anything: the same bits as the reference's loop nest, 8 bytes per element
 // less traffic.
@@ -417,7 +417,7 @@ __global__ void lbfgs_epilogue_kernel(const double *src, uint64_t count, Epilogu
 }
 
 // rho of pair j of the recursion (slot idx(j) of the ring), validity flags, alpha[j] = 0 for
-// invalid pairs (bridge_optimizer.m:1078-1081).
+// invalid pairs (bridge_optimizer.m:1067-1070).
 __global__ void lbfgs_prologue_kernel(const uintptr_t *rho_handles, int history_size, int history_count,
                                       int history_index, float *alpha, int *valid)
 {
@@ -711,7 +711,7 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers, uin
                                 float *step_size)
 try {
     // The reference performs no line search: the Wolfe constants and the losses are accepted
-    // and ignored (bridge_optimizer.m:1231-1233).
+    // and ignored (bridge_optimizer.m:1215-1216).
     (void)c1; (void)c2; (void)max_line_search; (void)current_loss; (void)prev_loss;
     Entry en;
     if (int rc = enter(device, buffer_sizes, num_weights, en)) return rc;
@@ -759,13 +759,13 @@ try {
 
     if (!valid.empty()) {
         const int count = (int)valid.size();
-        // q = -g (:1031-1043) stays in registers: the first dot product of the backward loop
+        // q = -g (:1025-1038) stays in registers: the first dot product of the backward loop
         {
             StreamArgs a = base;
             a.r0 = r.g; a.r1 = r.s(slot(valid[count - 1]), n);
             launch_dot(ctx, p, a, true);
         }
-        // backward loop, newest pair first (bridge_optimizer.m:1046-1137)
+        // backward loop, newest pair first (bridge_optimizer.m:1045-1130)
         for (int k = count - 1; k >= 0; k--) {
             const int j = valid[k], idx = slot(j);
             launch_reduction(ctx, p, Epilogue{kOpAlpha, rho_ptr(idx), alpha + j, nullptr, p.d_scalars});
@@ -781,7 +781,7 @@ try {
                 launch_stream<kModeAxpy, true>(ctx, p, a);
             }
         }
-        // forward loop, oldest pair first (:1143-1216)
+        // forward loop, oldest pair first (:1133-1201)
         for (int k = 0; k < count; k++) {
             const int j = valid[k], idx = slot(j);
             launch_reduction(ctx, p, Epilogue{kOpBeta, rho_ptr(idx), alpha + j, nullptr, p.d_scalars});
@@ -795,7 +795,7 @@ try {
             }
         }
     }
-    // p = -r (r = -g when no pair took part); x += a p; old_g = g; s_cur = a p  (:1219-1259), and with a
+    // p = -r (r = -g when no pair took part); x += a p; old_g = g; s_cur = a p  (:1203-1259), and with a
     // non-empty history y_prev = g - old_g, rho_prev = 0  (:1262-1310)
     {
         UpdateArgs u{};
@@ -824,7 +824,7 @@ int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffe
                                        float current_loss, float prev_loss, uintptr_t command_pool,
                                        float *step_size)
 {
-    // With or without a pool the reference runs the same code (bridge_optimizer.m:1365-1400).
+    // With or without a pool the reference runs the same code (bridge_optimizer.m:1356-1392).
     (void)command_pool;
     return execute_lbfgs_step_mpsgraph(device, weight_buffers, gradient_buffers, old_gradient_buffers,
                                        search_dir_buffers, s_vectors_flat, y_vectors_flat, rho_buffers,

@@ -181,7 +181,7 @@ int execute_nadam_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                 float learning_rate, float beta1, float beta2, float epsilon,
                                 float weight_decay, int step_count);
 
-/* bridge_optimizer.h:155-203 / .m:980-1404; prototypes bridge.go:296-343.  One L-BFGS step
+/* bridge_optimizer.h:155-203 / .m:980-1393; prototypes bridge.go:296-343.  One L-BFGS step
  * with the statement order of the reference's loop nest: q = -g; two-loop recursion over
  * the history pairs whose |rho| >= 1e-10 (H0 = I); p = -r; x += initial_step * p (no line
  * search: c1, c2, max_line_search and the losses are ignored, as in the reference);
@@ -207,7 +207,7 @@ int execute_lbfgs_step_mpsgraph(uintptr_t device, uintptr_t *weight_buffers,
                                 int history_size, int history_count, int history_index,
                                 float initial_step, float c1, float c2, int max_line_search,
                                 float current_loss, float prev_loss, float *step_size);
-/* bridge_optimizer.h:179-203 / .m:1338-1404: the same step (the pool is not used). */
+/* bridge_optimizer.h:179-203 / .m:1324-1393: the same step (the pool is not used). */
 int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *weight_buffers,
                                        uintptr_t *gradient_buffers,
                                        uintptr_t *old_gradient_buffers,

@@ -4,20 +4,20 @@
  * Restates execute_lbfgs_step_mpsgraph (cgo_bridge/bridge_optimizer.m:980-1321),
  * which is a plain CPU loop nest over unified-memory buffers, statement by
  * statement, including three properties of that code a reader may not expect:
- *   - the recursion starts from q = -g and ends with p = -r (:1026-1040, :1219-1229),
+ *   - the recursion starts from q = -g and ends with p = -r (:1025-1038, :1203-1213),
  *     so with an empty or invalid history the weights move by +initial_step * g;
  *   - the newest history slot is part of the two-loop recursion before its y and
- *     rho have been recomputed (the recomputation is step 6, :1279-1335);
- *   - the old gradient is overwritten with the current one (:1253-1255) before
- *     y = g - old_g is formed (:1303-1305), so y is all zeros for finite gradients
+ *     rho have been recomputed (the recomputation is step 6, :1242-1312);
+ *   - the old gradient is overwritten with the current one (:1237-1238) before
+ *     y = g - old_g is formed (:1285-1288), so y is all zeros for finite gradients
  *     and every rho the step itself writes is 0.
  * Every written floating-point operation rounds once to binary32 (build with
  * -ffp-contract=off).
  *
  * Dot products come in two evaluation orders:
  *   GM_ORACLE_DOT_REFERENCE  the reference's: fp32 running sum in element order
- *       (per tensor, tensors then added, for the recursion :1098-1103, :1176-1181;
- *       one running sum across all tensors for s.y, :1311-1313);
+ *       (per tensor, tensors then added, for the recursion :1100-1104, :1172-1176;
+ *       one running sum across all tensors for s.y, :1294-1297);
  *   GM_ORACLE_DOT_TREE       the HIP library's: exact fp64 products summed by a
  *       fixed radix-1024 tree in fp64, rounded once to fp32 at the end.
  * The tree (same for every dot): each tensor is cut into slices of 1024
@@ -101,11 +101,11 @@ static float dot_reference(const float *const *a, const float *const *b, const s
     float total = 0.0f;
     for (int t = 0; t < num_tensors; t++) {
         if (per_tensor) {
-            float dot = 0.0f;                                   /* :1098-1103 */
+            float dot = 0.0f;                                   /* :1100-1104 */
             for (size_t k = 0; k < n[t]; k++) dot += a[t][k] * b[t][k];
             total += dot;
         } else {
-            for (size_t k = 0; k < n[t]; k++) total += a[t][k] * b[t][k];   /* :1311-1313 */
+            for (size_t k = 0; k < n[t]; k++) total += a[t][k] * b[t][k];   /* :1294-1297 */
         }
     }
     return total;
@@ -127,11 +127,11 @@ int gm_oracle_lbfgs_step(float *const *w, const float *const *g, float *const *o
         history_index < 0 || history_index >= history_size)
         return -5;
 
-    /* step 1, :1026-1040: q = -g */
+    /* step 1, :1025-1038: q = -g */
     for (int i = 0; i < num_tensors; i++)
         for (size_t k = 0; k < n[i]; k++) dir[i][k] = -g[i][k];
 
-    /* step 2, first loop, :1046-1137 */
+    /* step 2, first loop, :1045-1130 */
     for (int j = history_count - 1; j >= 0; j--) {
         const int idx = (history_index - history_count + j + history_size) % history_size;
         const float rho_j = rho[idx];
@@ -148,7 +148,7 @@ int gm_oracle_lbfgs_step(float *const *w, const float *const *g, float *const *o
             for (size_t k = 0; k < n[i]; k++) dir[i][k] = dir[i][k] - alpha_j * yj[i][k];
     }
 
-    /* second loop, :1143-1216 (H0 = identity) */
+    /* second loop, :1133-1201 (H0 = identity) */
     for (int j = 0; j < history_count; j++) {
         const int idx = (history_index - history_count + j + history_size) % history_size;
         const float rho_j = rho[idx];
@@ -162,21 +162,21 @@ int gm_oracle_lbfgs_step(float *const *w, const float *const *g, float *const *o
             for (size_t k = 0; k < n[i]; k++) dir[i][k] = dir[i][k] + coeff * sj[i][k];
     }
 
-    /* step 3, :1219-1229: p = -r */
+    /* step 3, :1203-1213: p = -r */
     for (int i = 0; i < num_tensors; i++)
         for (size_t k = 0; k < n[i]; k++) dir[i][k] = -dir[i][k];
 
-    /* step 4, :1232-1233: fixed step */
+    /* step 4, :1215-1216: fixed step */
     const float a = initial_step;
     if (step_size) *step_size = a;
 
-    /* step 5, :1236-1256: x += a * p; old gradient <- current gradient */
+    /* step 5, :1219-1240: x += a * p; old gradient <- current gradient */
     for (int i = 0; i < num_tensors; i++) {
         for (size_t k = 0; k < n[i]; k++) w[i][k] = w[i][k] + a * dir[i][k];
         memcpy(old_g[i], g[i], n[i] * sizeof(float));
     }
 
-    /* step 6, :1259-1335 */
+    /* step 6, :1242-1312 */
     const int cur = history_index;
     for (int i = 0; i < num_tensors; i++)
         for (size_t k = 0; k < n[i]; k++) s[(size_t)cur * num_tensors + i][k] = a * dir[i][k];

@@ -180,7 +180,7 @@ def test_optimizer_sequence_from_fresh_state(dev):
 
 
 def test_non_finite_gradient(dev):
-    # inf - inf = NaN in y, NaN s.y fails the |s.y| > 1e-10 test, rho = 0 (bridge_optimizer.m:1322-1328)
+    # inf - inf = NaN in y, NaN s.y fails the |s.y| > 1e-10 test, rho = 0 (bridge_optimizer.m:1304-1310)
     sizes, m = [300, 5], 2
     rng = np.random.default_rng(9)
     st = seeded_state(rng, sizes, m, [2.0, 3.0])
@@ -246,7 +246,7 @@ def test_return_codes(dev):
 
     try:
         before = run.download()
-        assert call(device=0) == -1                                   # bridge_optimizer.m:1005-1009
+        assert call(device=0) == -1                                   # bridge_optimizer.m:1005-1008
         assert call(count=3) == -5 and call(index=2) == -5 and call(count=-1) == -5 and call(msize=0) == -5
         assert call(w=[run.w[0], 0]) == -8 and b"nil" in lib.gm_last_error()
         assert call(s=[0] + flat_s[1:]) == -8

@@ -34,7 +34,7 @@ def fresh_state(rng, sizes, m):
 
 @pytest.mark.parametrize("mode", [0, 1])
 def test_empty_history_moves_weights_by_plus_step_times_gradient(mode):
-    # q = -g, no recursion, p = -q = g, x += a * p  (bridge_optimizer.m:1026-1040, 1219-1250)
+    # q = -g, no recursion, p = -q = g, x += a * p  (bridge_optimizer.m:1025-1038, 1203-1240)
     rng = np.random.default_rng(1)
     sizes = [33, 1, 1500]
     st = fresh_state(rng, sizes, 3)
@@ -52,7 +52,7 @@ def test_empty_history_moves_weights_by_plus_step_times_gradient(mode):
 
 @pytest.mark.parametrize("mode", [0, 1])
 def test_rho_written_by_the_step_is_always_zero(mode):
-    # the old gradient is overwritten before y = g - old_g is formed (:1253-1255 before :1303-1305)
+    # the old gradient is overwritten before y = g - old_g is formed (:1237-1238 before :1285-1288)
     rng = np.random.default_rng(2)
     sizes, m = [40, 9], 3
     st = fresh_state(rng, sizes, m)
