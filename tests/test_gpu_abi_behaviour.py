@@ -112,16 +112,19 @@ def test_pooled_adam_and_queue_handles(dev, four):
     lib.release_command_queue(0)
 
 
-@pytest.mark.parametrize("chunk,nt,vec", [(0, 1, 2), (0, 1, 4), (0, 0, 1), (256, 1, 1), (1024, 0, 4),
-                                          (4096, 1, 2), (65536, 1, 4)])
-def test_launch_shape_variants_are_bit_identical(dev, chunk, nt, vec):
-    """Every selectable launch shape (lane width 1 / 2 / 4, chunk size, non-temporal hint) computes the
-    same bits, including on streams that are only 4-byte aligned (handles offset into a parent buffer)."""
+@pytest.mark.parametrize("chunk,nt,vec,lanes", [(0, 1, 2, 0), (0, 1, 4, 0), (0, 0, 1, 0), (256, 1, 1, 0), (1024, 0, 4, 0),
+                                                (4096, 1, 2, 0), (65536, 1, 4, 0), (0, 1, 1, 128), (256, 1, 1, 128),
+                                                (4096, 1, 2, 256), (0, 0, 4, 128), (0, 1, 0, 256), (0, 1, 0, 128)])
+def test_launch_shape_variants_are_bit_identical(dev, chunk, nt, vec, lanes):
+    """Every selectable launch shape (lane width 1 / 2 / 4, workgroups of 128 / 256 lanes, chunk size,
+    non-temporal hint) computes the same bits, including on streams that are only 4-byte aligned (handles
+    offset into a parent buffer)."""
     lib = dev.lib
     rng = np.random.default_rng(5)
     sizes = [1, 2, 3, 5, 255, 257, 1023, 4097, 70001, 262147]
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
     assert lib.gm_set_tuning(chunk, nt, vec) == 0
+    assert lib.gm_set_workgroup_lanes(lanes) == 0
     try:
         for rule, hyper in (("adam", ADAM), ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=0.0, nesterov=False)),
                             ("adadelta", dict(rho=0.9, eps=1e-6, weight_decay=0.0))):
@@ -130,7 +133,7 @@ def test_launch_shape_variants_are_bit_identical(dev, chunk, nt, vec):
                 grads = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
                 gpu.step(grads)
                 cpu.step(grads)
-            compare_snapshots(gpu.snapshot(), cpu.snapshot(), 0, f"{rule} chunk={chunk} nt={nt} vec={vec}")
+            compare_snapshots(gpu.snapshot(), cpu.snapshot(), 0, f"{rule} chunk={chunk} nt={nt} vec={vec} lanes={lanes}")
             gpu.close()
         # misaligned views: element 1 of each parent buffer (4-byte aligned only; not registry handles)
         n = 5000
@@ -151,6 +154,8 @@ def test_launch_shape_variants_are_bit_identical(dev, chunk, nt, vec):
             dev.free(h)
     finally:
         assert lib.gm_set_tuning(0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(0) == 0
+    assert lib.gm_set_workgroup_lanes(64) == -1 and lib.gm_set_workgroup_lanes(192) == -1
     assert lib.gm_set_tuning(1000, 1, 1) == -1 and lib.gm_set_tuning(0, 1, 3) == -1
     assert lib.gm_set_tuning(768, 1, 1) == -1          # 3 slices: not a power of two
 

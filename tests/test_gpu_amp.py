@@ -239,3 +239,29 @@ def test_async_steps_equal_the_synchronous_sequence(dev):
         for hs in g16_dev:
             for hd in hs:
                 dev.free(hd)
+
+
+@pytest.mark.parametrize("vec,lanes", [(2, 0), (4, 0), (1, 128), (2, 128), (4, 128)])
+def test_amp_launch_shape_variants_are_bit_identical(dev, vec, lanes):
+    """The mixed-precision step in every selectable lane width and workgroup size, over ragged sizes with an
+    overflow step in the middle: the same bits and the same skip / scale sequence as the oracle."""
+    lib = dev.lib
+    rng = np.random.default_rng(17)
+    sizes = [1, 2, 3, 7, 255, 257, 1023, 4097, 70001]
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    assert lib.gm_set_tuning(0, -1, vec) == 0
+    assert lib.gm_set_workgroup_lanes(lanes) == 0
+    try:
+        pair = AmpPair(dev, w, dict(HYPER, weight_decay=1e-4), (1024.0, 2.0, 0.5, 3))
+        try:
+            for t in range(6):
+                g16 = [(rng.normal(0, 1e-3, n) * 1024.0).astype(np.float16).view(np.uint16) for n in sizes]
+                if t == 2:
+                    g16[5][100] = 0x7C00          # +inf in one element of one tensor: the step is dropped
+                assert pair.step(g16) == (t == 2)
+                pair.compare(f"vec={vec} lanes={lanes} step={t}")
+        finally:
+            pair.close()
+    finally:
+        assert lib.gm_set_tuning(0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(0) == 0
