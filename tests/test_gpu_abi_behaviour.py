@@ -237,3 +237,30 @@ def test_ordering_against_a_callers_stream(dev):
         hip.hipHostFree(pin_out)
         dev.free(w)
         dev.free(gbuf)
+
+
+def test_gradient_handles_that_change_every_step(dev):
+    """A caller whose gradient buffers are new on every step (more distinct sets than the plan cache holds)
+    makes the library rebuild its chunk table each time and evict the oldest plan: every step stays exact."""
+    rng = np.random.default_rng(23)
+    sizes = [70001, 5, 4097, 262147, 1023]
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    gpu, cpu = GpuRun(dev, "adam", ADAM, w), OracleRun("adam", ADAM, w)
+    sets = 24
+    grads = [[rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes] for _ in range(sets)]
+    handles = [[dev.from_numpy(g) for g in gs] for gs in grads]
+    own = gpu.c_g
+    try:
+        for t in range(3 * sets):
+            k = (7 * t) % sets
+            gpu.c_g = pkg.handle_array(handles[k])
+            gpu.launch()
+            cpu.step(grads[k])
+            if t % 17 == 0 or t == 3 * sets - 1:
+                compare_snapshots(gpu.snapshot(), cpu.snapshot(), 0, f"step {t}")
+    finally:
+        gpu.c_g = own
+        gpu.close()
+        for hs in handles:
+            for h in hs:
+                dev.free(h)
