@@ -64,6 +64,18 @@ WORKLOADS = {
 }
 
 
+def cpu_model():
+    """The host CPU's model name (reported beside the CPU baseline)."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
+
+
 def time_steps(dev, launch, steps, warmup):
     """W untimed steps, then exactly K steps bracketed by a device synchronisation on both
     sides.  Returns (wall ms per step, HIP-event ms per launch)."""
@@ -119,7 +131,8 @@ def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_
     dt = time.perf_counter() - t0
     return {"value": total * steps / dt, "unit": "params/s", "cores": threads, "kind": "port",
             "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} steps in "
-                      f"{dt:.1f} s, oracle/oracle.c with OpenMP on {threads} threads"}
+                      f"{dt:.1f} s, oracle/oracle.c with OpenMP on {threads} threads of {os.cpu_count()} "
+                      f"({cpu_model()})"}
 
 
 LBFGS_WORKLOADS = {
@@ -302,7 +315,7 @@ def bench_primitives(args, pkg, dev):
         result["cpu_baseline"] = {"value": 6 * host_elems * reps / dt / 1e9, "unit": "GB/s", "cores": threads,
                                   "kind": "port",
                                   "sample": f"fp32->fp16 conversion of {host_elems} elements, {reps} calls in "
-                                            f"{dt:.1f} s, oracle/oracle.c on {threads} threads"}
+                                            f"{dt:.1f} s, oracle/oracle.c on {threads} threads ({cpu_model()})"}
     for h in (f32, f16, f32b):
         dev.free(h)
     dev.close()
@@ -336,7 +349,7 @@ def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
     return {"value": total * steps / dt, "unit": "params/s", "cores": 1, "kind": "port",
             "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} steps in {dt:.1f} s, "
                       "oracle/oracle_lbfgs.c in the reference's summation order on one thread (the reference "
-                      "runs this step as a single-threaded CPU loop)"}
+                      f"runs this step as a single-threaded CPU loop); host: {cpu_model()}"}
 
 
 def run_all(args):
