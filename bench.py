@@ -124,7 +124,7 @@ def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_
     t0 = time.perf_counter()
     run.step(g)
     one = max(time.perf_counter() - t0, 1e-4)
-    steps = int(min(2000, max(3, target_seconds / one)))
+    steps = int(min(1_000_000, max(3, target_seconds / one)))
     t0 = time.perf_counter()
     for _ in range(steps):
         run.step(g)
