@@ -323,7 +323,7 @@ def test_c5_size_dot_and_plain_step(dev):
         del a
         w0 = [dev.to_numpy(lists["w"][i], sizes[i]) for i in (0, 2, 33, 399)]
         step = ctypes.c_float()
-        # history_count 1 with rho = 0: update from the gradient, then the curvature pass
+        # history_count 1 with rho = 0: the update pass from the gradient, which also writes y_prev and rho_prev
         assert lib.execute_lbfgs_step_mpsgraph(D, arr(lists["w"]), arr(lists["g"]), arr(lists["old_g"]),
                                                arr(lists["dir"]), arr(lists["s"]), arr(lists["y"]), arr([rho]),
                                                alpha, n, bs, 1, 1, 0, 0.25, 1e-4, 0.9, 20, 0.0, 0.0,
