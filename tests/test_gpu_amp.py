@@ -265,3 +265,21 @@ def test_amp_launch_shape_variants_are_bit_identical(dev, vec, lanes):
     finally:
         assert lib.gm_set_tuning(0, -1, 0) == 0
         assert lib.gm_set_workgroup_lanes(0) == 0
+
+
+def test_amp_over_many_tiny_tensors(dev):
+    """400 tensors of 1 to 700 elements: 256-element chunks, so the overflow check runs one small workgroup per
+    chunk; an inf in the last element of the last tensor must still drop the whole step."""
+    rng = np.random.default_rng(43)
+    sizes = [int(x) for x in rng.integers(1, 701, 400)]
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    pair = AmpPair(dev, w, HYPER, (4096.0, 2.0, 0.5, 2))
+    try:
+        for t in range(5):
+            g16 = [(rng.normal(0, 1e-3, n) * 4096.0).astype(np.float16).view(np.uint16) for n in sizes]
+            if t == 1:
+                g16[-1][-1] = 0xFC00          # -inf
+            assert pair.step(g16) == (t == 1)
+        pair.compare("tiny tensors")
+    finally:
+        pair.close()

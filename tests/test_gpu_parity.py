@@ -138,6 +138,22 @@ def test_variants_and_ragged_edges(dev, rule, hyper):
              steps=6, check_every=3, nthreads=1)
 
 
+@pytest.mark.parametrize("rule,hyper", [
+    ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=0.0, nesterov=False)),
+    ("adagrad", dict(lr=0.01, eps=1e-10, weight_decay=0.0)),
+    ("adam", dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)),
+])
+def test_lists_of_many_tiny_tensors(dev, rule, hyper):
+    """Hundreds of tensors of 1 to 700 elements (biases, normalisation scales): the planner then cuts the list
+    into 256-element chunks, one descriptor per workgroup; with a few large tensors mixed in, into 1024."""
+    rng = np.random.default_rng(41)
+    for sizes in ([int(x) for x in rng.integers(1, 701, 400)],
+                  [int(x) for x in rng.integers(64, 513, 300)] + [200_000] * 12):
+        w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+        run_both(dev, rule, hyper, w, lambda k: [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes],
+                 steps=4, check_every=2, nthreads=1)
+
+
 SPECIALS = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-40, -3e-39, 1.17549435e-38,
                      3.4028235e38, -3.4028235e38, 1e-30, 1e30, 1.0, -1.0, 65504.0, 1e-8, 5e-324], dtype=np.float32)
 
