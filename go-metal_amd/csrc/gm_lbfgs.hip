@@ -19,8 +19,9 @@
 // non-finite g.  s_prev . y_prev is then a sum of zeros and NaNs, |s.y| > 1e-10 is false either
 // way, and rho_prev = 0 (:1304-1310), whatever s_prev holds.  The update pass therefore writes
 // y_prev = g - g from the gradient it already holds and rho_prev is set to 0 without reading
-// s_prev or summing anything: the same bits as the reference's loop nest, 8 bytes per element
-// less traffic.
+// s_prev or summing anything: the same bits as the reference's loop nest, 12 bytes per element
+// less traffic than a curvature pass of its own (read g, old_g, s_prev; write y_prev), 4 less
+// than a real dot product riding on the update pass.
 //
 // Which pairs are valid is read back once per step (history_count flags), so
 // only the passes that do work are launched; with the history the reference's
