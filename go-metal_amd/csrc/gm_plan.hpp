@@ -54,20 +54,31 @@ enum RuleKind : int {
     kRuleAdamAMP,
 };
 
+// A run of chunks of one size inside the table.  A list whose small tensors would leave many
+// workgroups of the list's chunk size idle gets a second segment with a smaller chunk size for
+// them; each segment is one launch of the update kernel.
+struct PlanSegment {
+    uint32_t first_chunk = 0;
+    uint32_t num_chunks = 0;
+    int chunk_elements = 0;
+};
+
 struct MultiTensorPlan {
     // ---- key ----
     int kind = 0;
     int variant = 0;             // rule-specific bits that change validation (e.g. which optional states are on)
     int num_tensors = 0;
     int requested_chunk_elements = 0;   // 0: chosen by the planner
-    int chunk_elements = 0;             // the size in force for this plan
+    int chunk_elements = 0;             // the size in force for this plan's first segment
     uint64_t generation = 0;
     std::vector<uintptr_t> handles;   // kNumSlots * num_tensors, slot-major
     std::vector<int> sizes;
     // ---- result ----
     int status = 0;              // validation result: 0 or the entry point's error code
     Chunk *d_chunks = nullptr;
-    uint32_t num_chunks = 0;
+    uint32_t num_chunks = 0;     // all segments together
+    PlanSegment segment[2];
+    int num_segments = 0;
     uint64_t total_elements = 0;
     ~MultiTensorPlan();
 };
