@@ -330,7 +330,9 @@ int gm_fill_normal_f16(uintptr_t device, uintptr_t buffer, size_t num_elements, 
 int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, size_t bytes);
 /* Launch-shape overrides for sweeps: elements per chunk (a power-of-two multiple of
  * 256 * vec, of 1024 when vec is automatic; 0 = default: 65536, 16384, 4096, 1024 or 256, the largest
- * that keeps idle workgroups under 5 % for the tensor list), non-temporal memory hints
+ * that keeps idle workgroups under 5 % for the tensor list, plus a smaller size for the list's
+ * small tensors when they would idle 16384 workgroups or more; a size given here applies to
+ * the whole list), non-temporal memory hints
  * on/off (-1 = default on) and fp32 elements per lane (1, 2 or 4; 0 = default: 2 for rules
  * with up to five streams, else 1).
  * -1 if the combination is not valid (nothing changes). */
