@@ -381,7 +381,7 @@ def main():
     ap.add_argument("--no-amp", action="store_true")
     ap.add_argument("--history", type=int, default=0, help="L-BFGS workloads: history size (default 10)")
     ap.add_argument("--rule", default="", choices=["", "sgd", "adam", "rmsprop", "adagrad", "adadelta", "nadam"],
-                    help="run another update rule (with BASELINE's hyper-parameters for it) over the workload's list")
+                    help="run another update rule (with the benchmark configurations' hyper-parameters for it) over the workload's list")
     # launch-shape overrides (gm_set_tuning) for comparing lane widths and chunk sizes; 0 / -1 = default
     ap.add_argument("--chunk", type=int, default=0, help="elements per chunk")
     ap.add_argument("--vec", type=int, default=0, help="fp32 elements per lane: 1, 2 or 4 (0: chosen per launch)")
