@@ -105,6 +105,7 @@ HOST_ABI = {
     "gmo_cleanup": (None, [u]),
     "gmo_get_state_json": (vp, [u]),
     "gmo_load_state_json": (i, [u, c_str]),
+    "gmo_state_json_normalize": (vp, [c_str]),
     "gmo_get_checkpoint_json": (vp, [u]),
     "gmo_load_checkpoint_json": (i, [u, c_str]),
     "gmo_get_field": (f, [u, c_str]),

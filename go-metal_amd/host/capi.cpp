@@ -316,6 +316,23 @@ try {
     return -1;
 }
 
+char *gmo_state_json_normalize(const char *json)
+try {
+    auto [state, perr] = OptimizerState::FromJSON(json ? json : "");
+    if (!perr.empty()) {
+        fail(perr);
+        return nullptr;
+    }
+    ok();
+    std::string js = state.ToJSON();
+    char *out = (char *)std::malloc(js.size() + 1);
+    if (out) std::memcpy(out, js.c_str(), js.size() + 1);
+    return out;
+} catch (...) {
+    note_exception();
+    return nullptr;
+}
+
 char *gmo_get_checkpoint_json(uintptr_t opt)
 try {
     if (!opt) { fail(Errorf("object handle is nil")); return nullptr; }

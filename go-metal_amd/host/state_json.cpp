@@ -298,6 +298,7 @@ std::pair<OptimizerState, Error> OptimizerState::FromJSON(const std::string &tex
                 }
                 if (!ps.expect('}')) return {st, ps.err};
             } else if (key == "state_data") {
+                st.StateData.clear();          // a repeated key replaces the slice, as encoding/json does
                 ps.ws();
                 if (ps.literal("null")) {
                     // Go writes a nil slice as null
@@ -367,6 +368,11 @@ std::pair<OptimizerState, Error> OptimizerState::FromJSON(const std::string &tex
         }
     }
     if (!ps.expect('}')) return {st, ps.err};
+    ps.ws();
+    if (ps.p != ps.end) {          // encoding/json: "invalid character ... after top-level value"
+        ps.fail("data after the top-level value");
+        return {st, ps.err};
+    }
     return {st, ""};
 }
 

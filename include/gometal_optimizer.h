@@ -64,6 +64,10 @@ void     gmo_cleanup(uintptr_t opt);
 char    *gmo_get_state_json(uintptr_t opt);
 /* LoadState(state) with state decoded from JSON (every number becomes a float64, as in Go). */
 int      gmo_load_state_json(uintptr_t opt, const char *json);
+/* Decodes an OptimizerState document and encodes it again (caller frees with gmo_free_string);
+ * NULL with gmo_last_error() set when the document does not decode.  No optimizer object and no
+ * GPU are involved: the serializer on its own, for tools and tests. */
+char    *gmo_state_json_normalize(const char *json);
 /* The same through the reference's JSON checkpoint document (checkpoints/checkpoint.go:38-52):
  * GetState() wrapped as {"model_spec", "weights", "training_state", "optimizer_state", "metadata"},
  * and LoadState() from the "optimizer_state" member of such a document. */
