@@ -338,6 +338,36 @@ def test_lr_schedulers_follow_the_reference_formulas(vanilla_sgd):
         lib.gmo_scheduler_free(h)
 
 
+def test_lr_schedulers_reference_tables():
+    """The known answers of the reference's own tests, with its tolerances (training/scheduler_test.go:8-108)."""
+    mk = lib.gmo_scheduler_new
+    step = mk(0, 2, 0.1, 0.0, None)                                   # TestStepLRScheduler
+    for epoch, want in [(0, 0.1), (1, 0.1), (2, 0.01), (3, 0.01), (4, 0.001), (5, 0.001), (6, 0.0001)]:
+        assert abs(lib.gmo_scheduler_get_lr(step, epoch, 0, 0.1) - want) <= 1e-8
+    expo = mk(1, 0, 0.9, 0.0, None)                                   # TestExponentialLRScheduler
+    for epoch, want in [(0, 0.1), (1, 0.09), (2, 0.081), (3, 0.0729), (4, 0.06561), (5, 0.059049)]:
+        assert abs(lib.gmo_scheduler_get_lr(expo, epoch, 0, 0.1) - want) <= 1e-8
+    cos = mk(2, 5, 0.0001, 0.0, None)                                 # TestCosineAnnealingLRScheduler
+    for epoch, want in [(0, 0.01), (5, 0.0001), (2, 0.006580)]:
+        assert abs(lib.gmo_scheduler_get_lr(cos, epoch, 0, 0.01) - want) <= 1e-6
+    assert lib.gmo_scheduler_get_lr(cos, 10, 0, 0.01) == 0.0001
+    plateau = mk(3, 2, 0.5, 0.01, b"min")                             # TestReduceLROnPlateauScheduler
+    lr = lib.gmo_scheduler_plateau_step(plateau, 1.0, 0.1)
+    assert lr == 0.1
+    lr = lib.gmo_scheduler_plateau_step(plateau, 0.98, lr)
+    assert lr == 0.1
+    lr = lib.gmo_scheduler_plateau_step(plateau, 0.99, lr)
+    assert lr == 0.1
+    lr = lib.gmo_scheduler_plateau_step(plateau, 0.99, lr)
+    assert lr == 0.05
+    names = [(mk(0, 10, 0.1, 0.0, None), b"StepLR"), (mk(1, 0, 0.9, 0.0, None), b"ExponentialLR"),
+             (mk(2, 10, 0.0, 0.0, None), b"CosineAnnealingLR"), (mk(3, 5, 0.5, 0.01, b"min"), b"ReduceLROnPlateau")]
+    for h, want in names:                                             # TestSchedulerNames (:111-128)
+        assert lib.gmo_scheduler_name(h) == want
+    for h in [step, expo, cos, plateau] + [h for h, _ in names]:
+        lib.gmo_scheduler_free(h)
+
+
 # ---- optimizer/lbfgs.go without a GPU: lbfgs_test.go:11-32, 131-162 and the Go error strings ----
 def test_lbfgs_default_config_and_constructor_errors(mm):
     cfg = pkg.HostLBFGS.default_config()
