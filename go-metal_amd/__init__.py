@@ -106,6 +106,12 @@ HOST_ABI = {
     "gmo_get_state_json": (vp, [u]),
     "gmo_load_state_json": (i, [u, c_str]),
     "gmo_state_json_normalize": (vp, [c_str]),
+    "gmo_extract_float32_param": (f, [c_str, c_str, f]),
+    "gmo_extract_bool_param": (i, [c_str, c_str, i]),
+    "gmo_extract_uint64_param": (ctypes.c_uint64, [c_str, c_str, ctypes.c_uint64]),
+    "gmo_validate_state_type": (i, [c_str, c_str]),
+    "gmo_restore_buffer_state": (i, [u, fp, i, i, c_str]),
+    "gmo_extract_buffer_state": (i, [u, i, c_str, c_str, fp, i]),
     "gmo_get_checkpoint_json": (vp, [u]),
     "gmo_load_checkpoint_json": (i, [u, c_str]),
     "gmo_get_field": (f, [u, c_str]),

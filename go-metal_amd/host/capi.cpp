@@ -48,6 +48,19 @@ std::vector<Pointer> pointers(const uintptr_t *p, int n)
     return v;
 }
 
+// The parameters object of an OptimizerState document, decoded as encoding/json would.
+std::map<std::string, ParamValue> parametersFrom(const char *parameters_json)
+{
+    const std::string doc = std::string("{\"type\":\"\",\"parameters\":") + (parameters_json ? parameters_json : "{}") + "}";
+    auto [state, err] = OptimizerState::FromJSON(doc);
+    if (!err.empty()) {
+        fail(err);
+        return {};
+    }
+    ok();
+    return state.Parameters;
+}
+
 // No exception may cross the C boundary (the caller is C, Go or Python): a failed allocation or a
 // standard-library error inside an entry point becomes that entry point's failure value, with the
 // reason in gmo_last_error().
@@ -974,6 +987,69 @@ try {
 float gmo_pow(float x, float y) { return optimizer::pow(x, y); }
 
 int gmo_extract_buffer_index(const char *name) { return extractBufferIndex(name ? name : ""); }
+
+float gmo_extract_float32_param(const char *parameters_json, const char *key, float default_value)
+try {
+    return extractFloat32Param(parametersFrom(parameters_json), key ? key : "", default_value);
+} catch (...) {
+    note_exception();
+    return default_value;
+}
+
+int gmo_extract_bool_param(const char *parameters_json, const char *key, int default_value)
+try {
+    return extractBoolParam(parametersFrom(parameters_json), key ? key : "", default_value != 0) ? 1 : 0;
+} catch (...) {
+    note_exception();
+    return default_value;
+}
+
+uint64_t gmo_extract_uint64_param(const char *parameters_json, const char *key, uint64_t default_value)
+try {
+    return extractUint64Param(parametersFrom(parameters_json), key ? key : "", default_value);
+} catch (...) {
+    note_exception();
+    return default_value;
+}
+
+int gmo_validate_state_type(const char *optimizer_type, const char *state_type)
+try {
+    OptimizerState state;
+    state.Type = state_type ? state_type : "";
+    Error e = validateStateType(optimizer_type ? optimizer_type : "", &state);
+    return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+int gmo_restore_buffer_state(uintptr_t buffer, const float *data, int num_elements, int buffer_size,
+                             const char *name)
+try {
+    std::vector<float> values;
+    if (data && num_elements > 0) values.assign(data, data + num_elements);
+    Error e = restoreBufferState(reinterpret_cast<Pointer>(buffer), values, buffer_size, name ? name : "");
+    return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+int gmo_extract_buffer_state(uintptr_t buffer, int buffer_size, const char *name, const char *state_type,
+                             float *data, int num_elements)
+try {
+    auto [tensor, err] = extractBufferState(reinterpret_cast<Pointer>(buffer), buffer_size, name ? name : "",
+                                            state_type ? state_type : "");
+    if (!err.empty()) return fail(err);
+    ok();
+    if (!tensor) return 0;
+    if (data)
+        for (int i = 0; i < num_elements && i < (int)tensor->Data.size(); i++) data[i] = tensor->Data[i];
+    return 1;
+} catch (...) {
+    note_exception();
+    return -1;
+}
 
 int gmo_calculate_tensor_size(const int *dims, int ndims)
 try {

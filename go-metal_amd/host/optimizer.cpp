@@ -38,7 +38,7 @@ Error validateStateType(const std::string &optimizerType, const OptimizerState *
     return "";
 }
 
-// optimizer/adam.go:142-148
+// optimizer/adam.go:237-251
 float pow(float x, float y)
 {
     if (y == 0) return 1.0f;
@@ -48,6 +48,7 @@ float pow(float x, float y)
     return result;
 }
 
+// optimizer/adam.go:142-148
 int calculateTensorSize(const std::vector<int> &shape)
 {
     int size = 1;

@@ -66,7 +66,7 @@ public:
     virtual void Cleanup() = 0;
 };
 
-// ---- helpers: optimizer/interface.go:56-84, state_helpers.go:14-74, adam.go:142-148 ----
+// ---- helpers: optimizer/interface.go:56-84, state_helpers.go:14-74, adam.go:142-148, 237-251 ----
 int extractBufferIndex(const std::string &name);
 Error validateStateType(const std::string &optimizerType, const OptimizerState *state);
 int calculateTensorSize(const std::vector<int> &shape);

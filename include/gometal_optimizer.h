@@ -154,6 +154,20 @@ double      gmo_scheduler_apply(uintptr_t scheduler, uintptr_t opt, int epoch, i
 float gmo_pow(float x, float y);                           /* pow, optimizer/adam.go:236-251 */
 int gmo_extract_buffer_index(const char *name);
 int gmo_calculate_tensor_size(const int *dims, int ndims);
+/* state_helpers.go:53-74 on a JSON object of parameters (numbers decode to float64, as through
+ * encoding/json): the value under key when it has the type the helper accepts, else the default. */
+float    gmo_extract_float32_param(const char *parameters_json, const char *key, float default_value);
+int      gmo_extract_bool_param(const char *parameters_json, const char *key, int default_value);
+uint64_t gmo_extract_uint64_param(const char *parameters_json, const char *key, uint64_t default_value);
+/* validateStateType, interface.go:79-84.  0, or -1 with the message in gmo_last_error(). */
+int gmo_validate_state_type(const char *optimizer_type, const char *state_type);
+/* restoreBufferState, state_helpers.go:34-50: 0, or -1 with the Go error string. */
+int gmo_restore_buffer_state(uintptr_t buffer, const float *data, int num_elements, int buffer_size,
+                             const char *name);
+/* extractBufferState, state_helpers.go:14-32: 1 when a tensor came back (its num_elements floats
+ * in data), 0 for a nil buffer (no tensor and no error), -1 with the Go error string. */
+int gmo_extract_buffer_state(uintptr_t buffer, int buffer_size, const char *name, const char *state_type,
+                             float *data, int num_elements);
 
 #ifdef __cplusplus
 }

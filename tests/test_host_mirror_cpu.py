@@ -433,3 +433,55 @@ def test_a_cpp_exception_stops_at_the_c_boundary(mm):
     h = lib.gmo_optimizer_new(pkg.KINDS["sgd"], cfg, dims, ndims, 1, mm, MOCK_DEVICE)
     assert h != 0
     lib.gmo_optimizer_free(h)
+
+
+# ---- optimizer/state_helpers_test.go restated: the tables of the reference's own tests
+@pytest.mark.parametrize("params,key,default,expected", [        # state_helpers_test.go:11-57
+    ({"learning_rate": 0.01}, "learning_rate", 0.001, 0.01),
+    ({"beta1": 0.9}, "learning_rate", 0.001, 0.001),
+    ({"learning_rate": "0.01"}, "learning_rate", 0.001, 0.001),
+    ({"learning_rate": 0.0}, "learning_rate", 0.001, 0.0),
+])
+def test_extract_float32_param(params, key, default, expected):
+    got = lib.gmo_extract_float32_param(json.dumps(params).encode(), key.encode(), default)
+    assert got == f32(expected)
+
+
+@pytest.mark.parametrize("params,key,default,expected", [        # state_helpers_test.go:60-106
+    ({"centered": True}, "centered", False, True),
+    ({"nesterov": True}, "centered", False, False),
+    ({"centered": "true"}, "centered", False, False),
+    ({"centered": False}, "centered", True, False),
+])
+def test_extract_bool_param(params, key, default, expected):
+    assert lib.gmo_extract_bool_param(json.dumps(params).encode(), key.encode(), int(default)) == int(expected)
+
+
+@pytest.mark.parametrize("params,key,default,expected", [        # state_helpers_test.go:109-163
+    ({"step_count": 100.0}, "step_count", 0, 100),
+    ({"learning_rate": 0.01}, "step_count", 0, 0),
+    ({"step_count": "100"}, "step_count", 0, 0),
+    ({"step_count": 0.0}, "step_count", 5, 0),
+    ({"step_count": 10.7}, "step_count", 0, 10),
+])
+def test_extract_uint64_param(params, key, default, expected):
+    assert lib.gmo_extract_uint64_param(json.dumps(params).encode(), key.encode(), default) == expected
+
+
+def test_extract_and_restore_buffer_state_messages():            # state_helpers_test.go:165-204
+    import ctypes
+    assert lib.gmo_extract_buffer_state(0, 64, b"test_buffer", b"momentum", None, 0) == 0     # nil: no tensor, no error
+    data = (ctypes.c_float * 2)(1.0, 2.0)
+    assert lib.gmo_restore_buffer_state(0, data, 2, 8, b"test_buffer") == -1
+    assert lib.gmo_last_error().decode() == "test_buffer buffer is nil"
+    assert lib.gmo_restore_buffer_state(MOCK_DEVICE, data, 2, 16, b"test_buffer") == -1
+    assert lib.gmo_last_error().decode() == "data size mismatch for test_buffer: expected 4 elements, got 2"
+
+
+@pytest.mark.parametrize("optimizer_type,state_type,ok", [       # state_helpers_test.go:260-308
+    ("Adam", "Adam", True), ("Adam", "SGD", False), ("Adam", "", False), ("", "Adam", False)])
+def test_validate_state_type(optimizer_type, state_type, ok):
+    rc = lib.gmo_validate_state_type(optimizer_type.encode(), state_type.encode())
+    assert (rc == 0) == ok
+    if not ok:                                                    # interface.go:81
+        assert lib.gmo_last_error().decode() == f"state type mismatch: expected {optimizer_type}, got {state_type}"
