@@ -150,6 +150,7 @@ HOST_ABI = {
     "gmo_tensor_convert_to": (u, [u, i]),
     "gmo_tensor_copy_float32_data": (i, [u, vp, i]),
     "gmo_tensor_to_float32_slice": (i, [u, vp, i]),
+    "gmo_tensor_string": (vp, [u]),
     "gmo_tensor_copy_from": (i, [u, u]),
     "gmo_calculate_size": (i, [ip, i, i]),
     "gmo_execute_step_with_precomputed_gradients": (i, [u, up, i, up, i]),

@@ -881,6 +881,22 @@ try {
     return -1;
 }
 
+char *gmo_tensor_string(uintptr_t tensor)
+try {
+    if (!tensor) {
+        fail(Errorf("object handle is nil"));
+        return nullptr;
+    }
+    ok();
+    const std::string text = T(tensor)->String();
+    char *out = (char *)std::malloc(text.size() + 1);
+    if (out) std::memcpy(out, text.c_str(), text.size() + 1);
+    return out;
+} catch (...) {
+    note_exception();
+    return nullptr;
+}
+
 int gmo_tensor_copy_from(uintptr_t dst, uintptr_t src)
 try {
     if (!dst) return fail(Errorf("object handle is nil"));

@@ -131,6 +131,7 @@ uintptr_t gmo_tensor_convert_to(uintptr_t tensor, int dtype);  /* ConvertTo, ten
 int       gmo_tensor_copy_float32_data(uintptr_t tensor, const float *data, int n);   /* tensor.go:189 */
 int       gmo_tensor_to_float32_slice(uintptr_t tensor, float *out, int capacity);    /* tensor.go:341; returns the element count */
 int       gmo_tensor_copy_from(uintptr_t dst, uintptr_t src);  /* CopyFrom, tensor.go:248 */
+char     *gmo_tensor_string(uintptr_t tensor);                 /* String, tensor.go:363-366; caller frees with gmo_free_string */
 int       gmo_calculate_size(const int *shape, int ndims, int dtype);                 /* tensor.go:137 */
 
 /* engine.ExecuteStepWithPrecomputedGradients (engine/training_engine.go:100-147) for any optimizer:

@@ -136,3 +136,47 @@ def test_execute_step_with_precomputed_gradients(env):
     for x in wt + gt:
         lib.gmo_tensor_release(x)
         lib.gmo_tensor_free(x)
+
+
+def test_tensor_string(env):                                  # memory_test.go:608-629 (skipped there: needs a GPU)
+    lib = env.lib
+    t = new_tensor(lib, [2, 3])
+    p = lib.gmo_tensor_string(t)
+    text = ctypes.string_at(p).decode()
+    lib.gmo_free_string(p)
+    assert text.startswith("Tensor{shape=[2 3], dtype=0, device=1, refs=1, gen=") and text.endswith("}")
+    lib.gmo_tensor_release(t)
+    lib.gmo_tensor_free(t)
+
+
+def test_tensor_with_a_zero_dimension(env):                   # memory_test.go:697-720 (skipped there)
+    lib = env.lib
+    t = new_tensor(lib, [0, 5])
+    assert lib.gmo_tensor_size(t) == 0
+    out = np.empty(4, np.float32)
+    assert lib.gmo_tensor_to_float32_slice(t, out.ctypes.data_as(vp), 4) < 0
+    assert lib.gmo_last_error().decode() == "tensor has invalid shape: [0 5]"       # tensor.go:352-354
+    lib.gmo_tensor_release(t)
+    lib.gmo_tensor_free(t)
+
+
+def test_reference_counting_from_many_threads(env):           # memory_test.go:417-455 (skipped there)
+    import threading
+    lib = env.lib
+    t = new_tensor(lib, [10, 10])
+    workers, rounds = 10, 100
+
+    def work():
+        for _ in range(rounds):
+            assert lib.gmo_tensor_retain(t) == t
+            lib.gmo_tensor_release(t)
+
+    threads = [threading.Thread(target=work) for _ in range(workers)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert lib.gmo_tensor_ref_count(t) == 1
+    lib.gmo_tensor_release(t)
+    assert lib.gmo_tensor_ref_count(t) == 0
+    lib.gmo_tensor_free(t)
