@@ -366,3 +366,32 @@ def test_dot_with_three_tree_levels(dev):
     finally:
         for h in ha + hb:
             dev.free(h)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_lists_histories_and_step_sizes(dev, seed):
+    """Tensor lists, ring sizes, history counts / indices, rho values (valid, zero, just under the 1e-10
+    threshold) and step sizes drawn from a seeded generator; three consecutive steps each, every buffer compared
+    bit for bit with the oracle in tree order."""
+    rng = np.random.default_rng(7000 + seed)
+    nt = int(rng.integers(1, 12))
+    sizes = [int(x) for x in np.exp(rng.uniform(0, np.log(300_000), nt)).astype(int)]
+    if rng.random() < 0.5:
+        sizes[int(rng.integers(0, nt))] = int(rng.choice([0, 1, 1023, 1024, 1025, 65536, 65537]))
+    m = int(rng.integers(1, 6))
+    count, index = int(rng.integers(0, m + 1)), int(rng.integers(0, m))
+    rho = [float(rng.choice([0.0, 5e-11, rng.normal(0, 20)])) for _ in range(m)]
+    st = seeded_state(rng, sizes, m, rho)
+    ref = clone(st)
+    run = LbfgsGpu(dev, st)
+    try:
+        for k in range(3):
+            g = [(rng.standard_normal(n) * 1e-2).astype(F) for n in sizes]
+            step = float(rng.choice([0.5, 1.0, 0.01]))
+            run.step(g, count, index, step)
+            rc, _ = oracle().lbfgs_step(ref, g, m, count, index, step, TREE)
+            assert rc == 0
+            assert_same_state(run.download(), ref, (seed, sizes, m, count, index, k))
+            index, count = (index + 1) % m, min(count + 1, m)
+    finally:
+        run.free()
