@@ -283,3 +283,28 @@ def test_amp_over_many_tiny_tensors(dev):
         pair.compare("tiny tensors")
     finally:
         pair.close()
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_lists_scales_and_injections(dev, seed):
+    """Tensor lists, initial scales, growth intervals, hyper-parameters and non-finite injections (+inf, -inf, two
+    NaN patterns) drawn from a seeded generator; eight steps each: the skip / scale sequence and every buffer agree
+    with the oracle bit for bit."""
+    rng = np.random.default_rng(9000 + seed)
+    nt = int(rng.integers(1, 10))
+    sizes = [int(x) for x in np.exp(rng.uniform(0, np.log(200_000), nt)).astype(int)]
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    hyper = dict(lr=float(10 ** rng.uniform(-4, -1)), beta1=0.9, beta2=0.999, eps=1e-8,
+                 weight_decay=float(rng.choice([0.0, 1e-4, 0.01])))
+    pair = AmpPair(dev, w, hyper, (float(2.0 ** rng.integers(0, 17)), 2.0, 0.5, int(rng.integers(1, 5))))
+    try:
+        for _ in range(8):
+            with np.errstate(all="ignore"):
+                g16 = [(rng.normal(0, 1e-3, n) * pair.st.scale).astype(np.float16).view(np.uint16) for n in sizes]
+            if rng.random() < 0.3:
+                k = int(rng.integers(0, nt))
+                g16[k][int(rng.integers(0, sizes[k]))] = int(rng.choice([0x7C00, 0xFC00, 0x7E00, 0xFFFF]))
+            pair.step(g16)
+        pair.compare(f"seed {seed}")
+    finally:
+        pair.close()
