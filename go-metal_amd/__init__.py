@@ -69,6 +69,7 @@ ABI = {
     "gm_amp_state_max_in_flight": (i, [u]),
     "execute_adam_amp_step_async": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, u]),
     "execute_adam_amp_step": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, i, u, ip, fp, ip]),
+    "gm_plan_cache_stats": (i, [u, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ip]),
     "gm_timer_start": (i, [u]),
     "gm_timer_stop": (f, [u]),
     "gm_fill_normal_f32": (i, [u, u, ctypes.c_size_t, ctypes.c_uint64, f, f]),

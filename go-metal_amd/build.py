@@ -26,6 +26,7 @@ HIPCC_FLAGS = [
 
 def sources():
     srcs = sorted(glob.glob(os.path.join(PKG_DIR, "csrc", "*.hip")))
+    srcs += sorted(glob.glob(os.path.join(PKG_DIR, "csrc", "*.cpp")))
     srcs += sorted(glob.glob(os.path.join(PKG_DIR, "host", "*.cpp")))
     return srcs
 

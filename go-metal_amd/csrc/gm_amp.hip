@@ -1,0 +1,490 @@
+// Mixed-precision (fp16-gradient) Adam step for gfx950: overflow check, update with fp16 weight
+// copy, loss-scale state machine; synchronous and run-ahead entry points.
+//
+// An inf in the last tensor must suppress the write to the first, and the Adam update is not
+// exactly invertible, so one pass cannot both check and write: the step is two streaming launches
+// plus a one-lane epilogue, all on one stream.
+#include "gm_launch.hpp"
+#include "gm_update_kernels.hpp"
+
+#include "../../include/gometal_hip.h"
+
+#include <cstring>
+
+namespace gm {
+
+constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
+
+// Loss-scale state machine, resident in HBM next to the tensors.
+struct alignas(16) AmpDeviceState {
+    // head: the 16 bytes every workgroup of the update kernel reads with one scalar load
+    float scale;
+    float inv_scale;        // 1.0f / scale, kept by whoever changes scale (IEEE division on host and device alike)
+    int found_inf;          // set by the check kernel, consumed and cleared by the epilogue
+    int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
+    // tail
+    int growth_tracker;
+    int last_skipped;
+    float growth_factor;
+    float backoff_factor;
+    int growth_interval;
+    int skipped_steps;      // steps dropped so far
+    int pad[2];
+};
+
+// Bias corrections for the asynchronous step.  The host does not know how many of the steps
+// still in flight were applied, so it sends the corrections (glibc powf, like every other
+// step) for each step count that is possible and the kernel picks by the device's count.
+constexpr int kAmpMaxInFlight = 8;
+struct AmpBiasTable {
+    int base;               // step count of entry 0 minus one: entry j is for t = base + 1 + j
+    int count;              // 1: use entry 0 whatever the device's count (synchronous step)
+    float bc1[kAmpMaxInFlight];
+    float bc2[kAmpMaxInFlight];
+};
+
+// Phase A: OR over every fp16 gradient element of "exponent field all ones"
+// (+-inf or NaN).  Per lane OR -> wavefront ballot -> one LDS word per wave ->
+// one atomic per workgroup that saw a hit.
+template <bool NT>
+__global__ void __launch_bounds__(kBlock)
+amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state)
+{
+    __shared__ unsigned int wave_hit[kBlock / 64];
+    const Chunk ch = chunks[blockIdx.x];
+    const unsigned short *g = reinterpret_cast<const unsigned short *>(ch.p[kSlotGrad]);
+    unsigned int bad = 0;
+    uint32_t done = 0;
+    if (ch.flags & kRecGrad16VectorOk) {
+        const uint32_t n8 = ch.count >> 3;
+        const uintx4 *g8 = reinterpret_cast<const uintx4 *>(g);
+        for (uint32_t base = threadIdx.x; base < n8; base += kBlock * kCheckUnroll) {
+            uintx4 v[kCheckUnroll];
+#pragma unroll
+            for (int u = 0; u < kCheckUnroll; u++) {
+                const uint32_t i = base + u * kBlock;
+                v[u] = (i < n8) ? stream_load<NT>(g8 + i) : uintx4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int u = 0; u < kCheckUnroll; u++) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const unsigned int e = v[u][c] & 0x7C007C00u;
+                    bad |= ((e & 0xFFFFu) == 0x7C00u) | ((e >> 16) == 0x7C00u);
+                }
+            }
+        }
+        done = n8 << 3;
+    }
+    for (uint32_t i = done + threadIdx.x; i < ch.count; i += kBlock)
+        bad |= ((stream_load<false>(g + i) & 0x7C00u) == 0x7C00u);
+
+    const unsigned long long ballot = __ballot(bad != 0);
+    if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = (ballot != 0ull);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned int any = 0;
+#pragma unroll
+        for (int k = 0; k < kBlock / 64; k++) any |= wave_hit[k];
+        if (any) atomicOr(&state->found_inf, 1);
+    }
+}
+
+// Phase B: the Adam update on unscaled gradients, skipped as a whole when the
+// flag is set.
+template <int VEC, bool NT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
+                       const AmpDeviceState *__restrict__ state, AmpBiasTable bias)
+{
+    // The state's head (scale, its reciprocal, flag, applied steps) comes with one 16-byte scalar load
+    // and the chunk descriptor with another, both issued before anything is decided; the bias
+    // table sits in the kernel arguments and its entry is picked by scalar selects.  No load
+    // waits for another except on the kernel-argument pointers themselves.
+    const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
+    const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
+    // (the weight pointer is never null; testing it here makes the compiler fetch the whole
+    // descriptor before the branch instead of the count first and the addresses after it)
+    if ((head.z != 0u) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
+        return;                                                        // step dropped, or an idle slice
+    const float inv_scale = __uint_as_float(head.y);
+    const int applied = (int)head.w;
+    int pick = bias.count > 1 ? applied - bias.base : 0;
+    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
+    float bc1 = bias.bc1[0], bc2 = bias.bc2[0];
+#pragma unroll
+    for (int j = 1; j < kAmpMaxInFlight; j++) {
+        if (pick == j) {
+            bc1 = bias.bc1[j];
+            bc2 = bias.bc2[j];
+        }
+    }
+    prm.bc1 = bc1;
+    prm.bc2 = bc2;
+    update_slice<AdamRule, VEC, NT, true, BLOCK>(ch, slice_shift, prm, inv_scale);
+}
+
+// Epilogue (one lane, same stream, after phase B has drained): advances the
+// loss-scale state machine and re-arms the flag.  A separate launch rather
+// than a last-workgroup ticket: a single counter bumped by every workgroup of
+// a 250k-workgroup grid serialises in the memory-side atomic unit.
+__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    AmpDeviceState st = *state;
+    const int found = st.found_inf;
+    if (found) {
+        st.scale = st.scale * st.backoff_factor;
+        st.growth_tracker = 0;
+        st.skipped_steps += 1;
+    } else {
+        st.applied_steps += 1;
+        st.growth_tracker += 1;
+        if (st.growth_tracker == st.growth_interval) {
+            st.scale = st.scale * st.growth_factor;
+            st.growth_tracker = 0;
+        }
+    }
+    st.inv_scale = 1.0f / st.scale;
+    st.last_skipped = found ? 1 : 0;
+    st.found_inf = 0;
+    *state = st;
+    // The post-state also goes straight into pinned host memory: the host reads it once the
+    // stream (or the event recorded after this launch) has completed, without a copy launch.
+    if (host_mirror) *host_mirror = st;
+}
+
+}  // namespace gm
+
+using namespace gm;
+
+extern "C" {
+
+// ---------------------------------------------------------- mixed precision --
+struct AmpState {
+    uint64_t magic;
+    Context *ctx;
+    AmpDeviceState *d_state;
+    AmpDeviceState *h_pinned;            // kAmpMaxInFlight + 1 slots: [0] synchronous read-backs, [1..] the ring
+    hipEvent_t ring_event[kAmpMaxInFlight];
+    // asynchronous steps: issue numbers count execute_adam_amp_step_async calls
+    uint64_t issued;                     // steps issued so far
+    uint64_t confirmed_issue;            // newest step whose post-state the host has seen
+    int confirmed_applied;               // the device's applied_steps after that step
+    int max_in_flight;                   // deepest run-ahead seen (diagnostics)
+};
+static const uint64_t kAmpMagic = 0x676D5F616D705F73ull;   // "gm_amp_s"
+
+static AmpState *amp_from_handle(uintptr_t h)
+{
+    if (h == 0) return nullptr;
+    auto *s = reinterpret_cast<AmpState *>(h);
+    return s->magic == kAmpMagic ? s : nullptr;
+}
+
+static bool amp_upload(AmpState *s)
+{
+    return hip_ok(hipMemcpyAsync(s->d_state, s->h_pinned, sizeof(AmpDeviceState),
+                                 hipMemcpyHostToDevice, s->ctx->stream), "amp state upload") &&
+           hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize");
+}
+
+// Waits for everything on the stream and reads the state back: afterwards no step is in flight.
+static bool amp_download(AmpState *s)
+{
+    if (!hip_ok(hipMemcpyAsync(s->h_pinned, s->d_state, sizeof(AmpDeviceState),
+                               hipMemcpyDeviceToHost, s->ctx->stream), "amp state download") ||
+        !hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize"))
+        return false;
+    s->confirmed_issue = s->issued;
+    s->confirmed_applied = s->h_pinned->applied_steps;
+    return true;
+}
+
+// Takes note of the asynchronous steps that have finished since the last look.  With
+// must_free_slot, blocks until at most kAmpMaxInFlight - 2 steps are unconfirmed, so that the
+// next step's bias table and ring slot are available.
+static bool amp_poll(AmpState *s, bool must_free_slot)
+{
+    for (;;) {
+        while (s->confirmed_issue < s->issued) {
+            const uint64_t next = s->confirmed_issue + 1;
+            const hipError_t q = hipEventQuery(s->ring_event[next % kAmpMaxInFlight]);
+            if (q == hipErrorNotReady) {
+                (void)hipGetLastError();     // "not ready" is an answer, not a failure to report later
+                break;
+            }
+            if (!hip_ok(q, "hipEventQuery")) return false;
+            s->confirmed_issue = next;
+            s->confirmed_applied = s->h_pinned[1 + next % kAmpMaxInFlight].applied_steps;
+        }
+        if (!must_free_slot || s->issued - s->confirmed_issue <= (uint64_t)kAmpMaxInFlight - 2) return true;
+        const uint64_t oldest = s->confirmed_issue + 1;
+        if (!hip_ok(hipEventSynchronize(s->ring_event[oldest % kAmpMaxInFlight]), "hipEventSynchronize"))
+            return false;
+    }
+}
+
+static void amp_free(AmpState *s)
+{
+    if (s->d_state) (void)hipFree(s->d_state);
+    if (s->h_pinned) (void)hipHostFree(s->h_pinned);
+    for (hipEvent_t e : s->ring_event)
+        if (e) (void)hipEventDestroy(e);
+    s->magic = 0;
+    delete s;
+}
+
+uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_factor,
+                              float backoff_factor, int growth_interval)
+try {
+    clear_error();
+    if (device == 0) return 0;
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return 0;
+    auto *s = new AmpState{};
+    s->magic = kAmpMagic;
+    s->ctx = ctx;
+    bool ok = hip_ok(hipMalloc(&s->d_state, sizeof(AmpDeviceState)), "hipMalloc(amp state)") &&
+              hip_ok(hipHostMalloc(&s->h_pinned, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState),
+                                   hipHostMallocDefault), "hipHostMalloc(amp state)");
+    for (int k = 0; ok && k < kAmpMaxInFlight; k++)
+        ok = hip_ok(hipEventCreateWithFlags(&s->ring_event[k], hipEventDisableTiming), "hipEventCreate");
+    if (ok) {
+        std::memset(s->h_pinned, 0, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState));
+        s->h_pinned->scale = init_scale;
+        s->h_pinned->inv_scale = 1.0f / init_scale;
+        s->h_pinned->growth_factor = growth_factor;
+        s->h_pinned->backoff_factor = backoff_factor;
+        s->h_pinned->growth_interval = growth_interval;
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        ok = amp_upload(s);
+    }
+    if (!ok) {
+        amp_free(s);
+        return 0;
+    }
+    return reinterpret_cast<uintptr_t>(s);
+} catch (...) {
+    note_exception();
+    return 0;
+}
+
+void gm_amp_state_destroy(uintptr_t amp_state)
+try {
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return;
+    make_current(s->ctx);
+    (void)hipStreamSynchronize(s->ctx->stream);     // ring copies may still be in flight
+    amp_free(s);
+} catch (...) {
+    note_exception();
+}
+
+int gm_amp_state_get(uintptr_t amp_state, float *scale, int *growth_tracker)
+{
+    return gm_amp_state_query(amp_state, scale, growth_tracker, nullptr, nullptr);
+}
+
+int gm_amp_state_query(uintptr_t amp_state, float *scale, int *growth_tracker, int *applied_steps,
+                       int *skipped_steps)
+try {
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    if (scale) *scale = s->h_pinned->scale;
+    if (growth_tracker) *growth_tracker = s->h_pinned->growth_tracker;
+    if (applied_steps) *applied_steps = s->h_pinned->applied_steps;
+    if (skipped_steps) *skipped_steps = s->h_pinned->skipped_steps;
+    return 0;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int gm_amp_state_max_in_flight(uintptr_t amp_state)
+{
+    AmpState *s = amp_from_handle(amp_state);
+    return s ? s->max_in_flight : -16;
+}
+
+int gm_amp_state_set(uintptr_t amp_state, float scale, int growth_tracker)
+try {
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    s->h_pinned->scale = scale;
+    s->h_pinned->inv_scale = 1.0f / scale;
+    s->h_pinned->growth_tracker = growth_tracker;
+    return amp_upload(s) ? 0 : -6;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int gm_amp_state_set_step_count(uintptr_t amp_state, int applied_steps)
+try {
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (applied_steps < 0) return -5;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    s->h_pinned->applied_steps = applied_steps;
+    if (!amp_upload(s)) return -6;
+    s->confirmed_applied = applied_steps;
+    return 0;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+// Plan, parameters and the three launches shared by the synchronous and the asynchronous step.
+static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffers,
+                       uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                       uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
+                       int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
+                       float weight_decay, int step_count, bool async, Launch &l,
+                       std::unique_lock<std::mutex> &lock)
+{
+    PlanRequest req{};
+    req.kind = kRuleAdamAMP;
+    req.num_tensors = num_weights;
+    req.slot[kSlotWeight] = weight_buffers;
+    req.slot[kSlotGrad] = gradient16_buffers;
+    req.slot[kSlotState0] = momentum_buffers;
+    req.slot[kSlotState1] = variance_buffers;
+    req.slot[kSlotWeight16] = weight16_buffers;
+    req.sizes = buffer_sizes;
+    req.required_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0) | (1u << kSlotState1);
+    req.missing_code = -4;
+    req.half_mask = (1u << kSlotGrad) | (1u << kSlotWeight16);
+    if (int rc = prepare(device, req, -6, l, lock)) return rc;
+    if (l.ctx != amp->ctx) {
+        set_error("the loss-scale state belongs to another device context");
+        return -16;
+    }
+
+    StepParams p = zero_params();
+    p.lr = learning_rate;
+    p.beta1 = beta1;
+    p.beta2 = beta2;
+    p.one_minus_beta1 = 1.0f - beta1;
+    p.one_minus_beta2 = 1.0f - beta2;
+    p.eps = epsilon;
+    p.weight_decay = weight_decay;
+
+    // The context lock is held from here on: the issue counters of the loss-scale state are
+    // only read and advanced under it.  An asynchronous step's post-state goes into the ring
+    // slot of its issue number, a synchronous step's into slot 0.
+    AmpDeviceState *host_mirror = amp->h_pinned;
+    AmpBiasTable bias{};
+    if (async) {
+        if (!amp_poll(amp, true)) return -6;
+        host_mirror = &amp->h_pinned[1 + (amp->issued + 1) % kAmpMaxInFlight];
+        const int in_flight = (int)(amp->issued - amp->confirmed_issue);
+        if (in_flight > amp->max_in_flight) amp->max_in_flight = in_flight;
+        bias.base = amp->confirmed_applied;
+        bias.count = in_flight + 1;
+        for (int j = 0; j <= in_flight; j++)
+            gm_bias_corrections(beta1, beta2, amp->confirmed_applied + 1 + j, &bias.bc1[j], &bias.bc2[j]);
+    } else {
+        bias.count = 1;
+        gm_bias_corrections(beta1, beta2, step_count, &bias.bc1[0], &bias.bc2[0]);
+    }
+
+    const uint32_t chunks = l.plan->num_chunks;
+    hipStream_t st = l.ctx->stream;
+    if (chunks > 0) {
+        int vec = current_vec();
+        if (vec == 0) vec = auto_vec(8);
+        const bool nt = current_nontemporal();
+        int block = current_block();
+        if (block == 0) block = auto_block(8);
+        SegmentLaunch seg[2];
+        int count;
+        if (!launch_geometry(*l.plan, vec, block, seg, count)) return -6;
+        // the check walks the whole table, one workgroup per chunk of either segment
+        if (nt) amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
+        else amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
+#define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, amp->d_state, bias)
+#define GM_LAUNCH_AMP_B(B)                                                              \
+        if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true, B); else GM_LAUNCH_AMP(4, false, B); }        \
+        else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true, B); else GM_LAUNCH_AMP(2, false, B); }   \
+        else { if (nt) GM_LAUNCH_AMP(1, true, B); else GM_LAUNCH_AMP(1, false, B); }
+        for (int s = 0; s < count; s++) {
+            const SegmentLaunch &g = seg[s];
+            if (block == 128) { GM_LAUNCH_AMP_B(128) } else { GM_LAUNCH_AMP_B(kBlock) }
+        }
+#undef GM_LAUNCH_AMP_B
+#undef GM_LAUNCH_AMP
+    }
+    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror);
+    return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
+}
+
+int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
+                          uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                          uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                          int num_weights, int *buffer_sizes, float learning_rate, float beta1,
+                          float beta2, float epsilon, float weight_decay, int step_count,
+                          uintptr_t amp_state, int *skipped, float *scale_out,
+                          int *growth_tracker_out)
+try {
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = amp_enqueue(device, amp, weight_buffers, gradient16_buffers, momentum_buffers,
+                             variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
+                             beta1, beta2, epsilon, weight_decay, step_count, false, l, lock))
+        return rc;
+    if (!hip_ok(hipStreamSynchronize(l.ctx->stream), "hipStreamSynchronize")) return -6;
+    amp->confirmed_issue = amp->issued;
+    amp->confirmed_applied = amp->h_pinned->applied_steps;
+    if (skipped) *skipped = amp->h_pinned->last_skipped;
+    if (scale_out) *scale_out = amp->h_pinned->scale;
+    if (growth_tracker_out) *growth_tracker_out = amp->h_pinned->growth_tracker;
+    return 0;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
+                                uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                                uintptr_t *variance_buffers, uintptr_t *weight16_buffers,
+                                int num_weights, int *buffer_sizes, float learning_rate, float beta1,
+                                float beta2, float epsilon, float weight_decay, uintptr_t amp_state)
+try {
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    if (int rc = amp_enqueue(device, amp, weight_buffers, gradient16_buffers, momentum_buffers,
+                             variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
+                             beta1, beta2, epsilon, weight_decay, 0, true, l, lock))
+        return rc;
+    // the event marks the arrival of this step's post-state in its ring slot
+    const uint64_t issue = amp->issued + 1;
+    const int slot = (int)(issue % kAmpMaxInFlight);
+    if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
+        // the step itself is enqueued; resynchronise the bookkeeping with the device
+        (void)amp_download(amp);
+        return -6;
+    }
+    amp->issued = issue;
+    return 0;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+}  // extern "C"

@@ -27,6 +27,7 @@ void note_exception() noexcept;
 bool hip_ok(hipError_t e, const char *what);
 
 struct MultiTensorPlan;
+struct TableSlot;
 
 // Large host <-> device copies of ordinary (pageable) host memory go through pinned staging
 // slots, two lanes at a time: each lane owns a stream, two slots and their events, moves one
@@ -47,6 +48,9 @@ struct Context {
     std::atomic<int> refs{0};
     std::mutex mu;                                    // guards plans and launches
     std::vector<std::unique_ptr<MultiTensorPlan>> plans;  // most recently used first
+    std::vector<TableSlot> free_tables;               // chunk-table slots of dropped plans, kept for reuse
+    std::atomic<uint64_t> plan_builds{0};             // chunk tables laid out so far (diagnostics)
+    std::atomic<uint64_t> table_allocations{0};       // table slots allocated so far (diagnostics)
     std::mutex stage_mu;                              // one staged copy at a time
     bool stage_ready = false;
     StageLane stage[kStageLanes];                     // created on first use, kept until the process ends
@@ -70,9 +74,11 @@ void registry_add(uintptr_t buffer, size_t bytes);
 void registry_remove(uintptr_t buffer);
 // 0 when the handle is not one of ours.
 size_t registry_length(uintptr_t buffer);
-// Bumped on every removal; cached launch plans are only valid for the
-// generation they were built in (a freed address may come back with a
-// different length).
-uint64_t registry_generation();
+
+// A freed address may come back with a different length, so whatever was validated against the
+// old allocation must be forgotten: deallocate_metal_buffer calls these (holding ctx->mu) with
+// the freed range.  Only the cached plans that hold a handle inside the range are affected.
+void plans_forget_range(Context *ctx, uintptr_t begin, size_t bytes);    // multi-tensor plans: dropped
+void lbfgs_forget_range(uintptr_t begin, size_t bytes);                  // L-BFGS plans: handles revalidated
 
 }  // namespace gm

@@ -47,7 +47,7 @@
 
 namespace gm {
 
-bool current_nontemporal();   // gm_multi_tensor.hip
+bool current_nontemporal();   // gm_plan_cache.hip
 
 namespace {
 
@@ -83,7 +83,6 @@ struct Epilogue {
 struct Plan {
     // key
     std::vector<int> sizes;
-    uint64_t generation = 0;
     // geometry
     LbChunk *d_chunks = nullptr;
     uint32_t num_chunks = 0;
@@ -499,20 +498,14 @@ bool ensure_geometry(Context *ctx, Plan &p, const int *sizes, int n)
 Plan *find_plan(Context *ctx, const int *sizes, int n)
 {
     auto &cache = plan_cache();
-    const uint64_t gen = registry_generation();
     for (size_t i = 0; i < cache.size(); i++) {
         Plan &p = *cache[i];
         if ((int)p.sizes.size() == n && std::memcmp(p.sizes.data(), sizes, (size_t)n * sizeof(int)) == 0) {
-            if (p.generation != gen) {       // handles may have been freed and reissued: revalidate
-                p.handles_valid = false;
-                p.generation = gen;
-            }
             if (i != 0) std::rotate(cache.begin(), cache.begin() + i, cache.begin() + i + 1);
             return cache[0].get();
         }
     }
     auto plan = std::make_unique<Plan>();
-    plan->generation = gen;
     if (!ensure_geometry(ctx, *plan, sizes, n)) return nullptr;
     if (cache.size() >= kMaxPlans) {
         (void)hipStreamSynchronize(ctx->stream);    // an evicted plan's scratch may still be in use
@@ -696,6 +689,18 @@ int enter(uintptr_t device, const int *sizes, int n, Entry &out)
 }
 
 }  // namespace
+
+// A buffer of the library was freed: plans that hold a handle inside it validate and upload
+// their handle table again on their next step (the address may come back with another length).
+void lbfgs_forget_range(uintptr_t begin, size_t bytes)
+{
+    const uintptr_t end = begin + bytes;
+    auto inside = [&](uintptr_t x) { return x >= begin && x < end; };
+    for (auto &p : plan_cache())
+        if (inside(p->alpha_handle) || std::any_of(p->handles.begin(), p->handles.end(), inside))
+            p->handles_valid = false;
+}
+
 }  // namespace gm
 
 using namespace gm;

@@ -85,7 +85,6 @@ bool make_current(Context *ctx) { return hip_ok(hipSetDevice(ctx->device_id), "h
 // -------------------------------------------------------------- registry ----
 static std::mutex g_reg_mu;
 static std::unordered_map<uintptr_t, size_t> g_reg;
-static std::atomic<uint64_t> g_reg_generation{1};
 
 void registry_add(uintptr_t buffer, size_t bytes)
 {
@@ -97,7 +96,6 @@ void registry_remove(uintptr_t buffer)
 {
     std::lock_guard<std::mutex> lk(g_reg_mu);
     g_reg.erase(buffer);
-    g_reg_generation.fetch_add(1);
 }
 
 size_t registry_length(uintptr_t buffer)
@@ -106,8 +104,6 @@ size_t registry_length(uintptr_t buffer)
     auto it = g_reg.find(buffer);
     return it == g_reg.end() ? 0 : it->second;
 }
-
-uint64_t registry_generation() { return g_reg_generation.load(); }
 
 // --------------------------------------------------------------- kernels ----
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -441,10 +437,17 @@ try {
 void deallocate_metal_buffer(uintptr_t buffer)
 try {
     if (buffer == 0) return;
-    if (registry_length(buffer) == 0) return;   // not ours (or already freed): leave it alone
-    registry_remove(buffer);
+    const size_t len = registry_length(buffer);
+    if (len == 0) return;   // not ours (or already freed): leave it alone
     Context *ctx = default_context();
-    if (ctx) make_current(ctx);
+    if (ctx) {
+        make_current(ctx);
+        // plans validated against this allocation go before the address can be handed out again
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        plans_forget_range(ctx, buffer, len);
+        lbfgs_forget_range(buffer, len);
+    }
+    registry_remove(buffer);
     (void)hipFree(reinterpret_cast<void *>(buffer));   // hipFree waits for work in flight
 } catch (...) {
     note_exception();

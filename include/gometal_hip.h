@@ -312,6 +312,13 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
 int gm_lbfgs_dot(uintptr_t device, uintptr_t *a_buffers, uintptr_t *b_buffers, int num_tensors,
                  int *buffer_sizes, float *result);
 
+/* Diagnostics of the plan cache behind the multi-tensor steps: chunk tables laid out so far
+ * (a step whose list and handles were seen before builds none), table slots allocated so far
+ * (device table + pinned host twin; dropped plans hand theirs on, so the count stops growing once
+ * the working set of lists has been seen) and plans currently cached.  Pointers may be NULL. */
+int gm_plan_cache_stats(uintptr_t device, uint64_t *plan_builds, uint64_t *table_allocations,
+                        int *cached_plans);
+
 /* Measurement helpers used by the benchmark and the profiles. */
 
 /* Records a start / stop event pair on the device's stream; gm_timer_stop
