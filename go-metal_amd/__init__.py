@@ -69,6 +69,7 @@ ABI = {
     "gm_amp_state_max_in_flight": (i, [u]),
     "execute_adam_amp_step_async": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, u]),
     "execute_adam_amp_step": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, i, u, ip, fp, ip]),
+    "execute_adam_step_noalloc": (i, [u, up, up, up, up, i, ip, f, f, f, f, f, i]),
     "gm_plan_cache_stats": (i, [u, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ip]),
     "gm_timer_start": (i, [u]),
     "gm_timer_stop": (f, [u]),

@@ -51,6 +51,7 @@ struct Context {
     std::vector<TableSlot> free_tables;               // chunk-table slots of dropped plans, kept for reuse
     std::atomic<uint64_t> plan_builds{0};             // chunk tables laid out so far (diagnostics)
     std::atomic<uint64_t> table_allocations{0};       // table slots allocated so far (diagnostics)
+    void *noalloc_scratch = nullptr;                  // this GPU's address of the allocation-free step's table
     std::mutex stage_mu;                              // one staged copy at a time
     bool stage_ready = false;
     StageLane stage[kStageLanes];                     // created on first use, kept until the process ends
@@ -80,5 +81,9 @@ size_t registry_length(uintptr_t buffer);
 // the freed range.  Only the cached plans that hold a handle inside the range are affected.
 void plans_forget_range(Context *ctx, uintptr_t begin, size_t bytes);    // multi-tensor plans: dropped
 void lbfgs_forget_range(uintptr_t begin, size_t bytes);                  // L-BFGS plans: handles revalidated
+
+// Resolves this GPU's address of the allocation-free step's descriptor table (a __device__
+// array) once, at context creation, with the device current.  false: error recorded.
+bool noalloc_bind_scratch(Context *ctx);
 
 }  // namespace gm

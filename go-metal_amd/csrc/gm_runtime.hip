@@ -64,7 +64,8 @@ Context *default_context()
         if (!hip_ok(hipSetDevice(0), "hipSetDevice") ||
             !hip_ok(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking), "hipStreamCreate") ||
             !hip_ok(hipEventCreate(&ctx->ev_start), "hipEventCreate") ||
-            !hip_ok(hipEventCreate(&ctx->ev_stop), "hipEventCreate")) {
+            !hip_ok(hipEventCreate(&ctx->ev_stop), "hipEventCreate") ||
+            !noalloc_bind_scratch(ctx)) {
             delete ctx;
             return;
         }

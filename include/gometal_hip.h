@@ -307,6 +307,22 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
                                 float beta1, float beta2, float epsilon, float weight_decay,
                                 uintptr_t amp_state);
 
+/* execute_adam_step_mpsgraph for callers that cannot allocate.  No counterpart in the reference:
+ * it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc.  Same arguments, arithmetic, update kernel and results as execute_adam_step_mpsgraph;
+ * the chunk table lives in a __device__ array of the library (2 MiB per GPU, held until the
+ * process ends) and is written by a kernel from tensor records passed as kernel arguments, so the
+ * call performs no hipMalloc, hipFree, copy or other allocating routine and never waits for the
+ * device.  Limits: 4096 tensors and 32768 chunk descriptors (about 2.1e9 parameters in chunks of
+ * 65536 elements); beyond them -17 and a message in gm_last_error, nothing launched.  Every call on
+ * a GPU rewrites that GPU's one table: calls are ordered on the library's stream, and calls that
+ * overlap on one GPU by any other means race.
+ * -1 device 0; -3 no GPU; -4 a required handle is 0 (nothing updated); -6 HIP error; -17 over the limits. */
+int execute_adam_step_noalloc(uintptr_t device, uintptr_t *weight_buffers, uintptr_t *gradient_buffers,
+                              uintptr_t *momentum_buffers, uintptr_t *variance_buffers, int num_weights,
+                              int *buffer_sizes, float learning_rate, float beta1, float beta2,
+                              float epsilon, float weight_decay, int step_count);
+
 /* The dot product of two tensor lists exactly as the L-BFGS step forms it (fp64 tree,
  * one rounding to fp32).  Synchronises.  Codes as execute_lbfgs_step_mpsgraph. */
 int gm_lbfgs_dot(uintptr_t device, uintptr_t *a_buffers, uintptr_t *b_buffers, int num_tensors,
