@@ -49,3 +49,12 @@ def transformer_block_sizes():
     sizes += [4096 * 4096] * 4
     assert len(sizes) == 400 and sum(sizes) == 1_012_301_824
     return sizes
+
+
+def two_segment_sizes():
+    """A list the planner cuts into two segments: one 120M-element tensor keeps 65536-element chunks within
+    the 5 % idle limit, and 80 small tensors in the middle of the list would idle about 20k workgroups of that
+    size, more than the 16384 that earn them a segment with a smaller chunk."""
+    small = [1, 255, 256, 257, 1023, 1025, 4095, 4097, 5, 300, 77, 2049] * 7
+    small = small[:80]
+    return small[:40] + [120_000_001] + small[40:]
