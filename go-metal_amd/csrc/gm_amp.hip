@@ -13,6 +13,8 @@
 
 namespace gm {
 
+constexpr float kMinLossScale = 1.17549435e-38f;   // FLT_MIN
+constexpr float kMaxLossScale = 3.40282347e+38f;   // FLT_MAX
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 
 // Loss-scale state machine, resident in HBM next to the tensors.
@@ -134,15 +136,21 @@ __global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     AmpDeviceState st = *state;
     const int found = st.found_inf;
+    // The scale stays a normal, finite fp32 number whatever the run does: a growth that would
+    // overflow to infinity (about 112 uninterrupted growth intervals from 65536) and a backoff
+    // that would leave the normal range are not applied.  Unbounded, the scale would stick at
+    // +inf (inf * 0.5 = inf) with a reciprocal of 0, or reach 0 with a reciprocal of +inf.
     if (found) {
-        st.scale = st.scale * st.backoff_factor;
+        const float next = st.scale * st.backoff_factor;
+        if (next >= kMinLossScale) st.scale = next;
         st.growth_tracker = 0;
         st.skipped_steps += 1;
     } else {
         st.applied_steps += 1;
         st.growth_tracker += 1;
         if (st.growth_tracker == st.growth_interval) {
-            st.scale = st.scale * st.growth_factor;
+            const float next = st.scale * st.growth_factor;
+            if (next <= kMaxLossScale) st.scale = next;
             st.growth_tracker = 0;
         }
     }

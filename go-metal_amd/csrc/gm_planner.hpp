@@ -127,6 +127,38 @@ struct PlanLayout {
 // Lays the request out.  requested_chunk > 0 fixes one chunk size for the whole list.
 void layout_plan(const PlanRequest &r, int requested_chunk, BufferLengthFn length_of, PlanLayout &out);
 
+#if defined(__HIPCC__)
+#define GM_HOST_DEVICE __host__ __device__
+#else
+#define GM_HOST_DEVICE
+#endif
+
+// One lane's share of a chunk: elements [first, first + count) of every stream.  `grouped`: the
+// share is one aligned vec-wide access per stream; otherwise its elements are accessed one by one
+// (a chunk's tail, or streams whose handles are not aligned for vec-wide lanes).  count == 0: the
+// lane lies past the chunk's end.  The update kernels and the CPU bounds harness both index
+// through this function.
+struct LaneShare {
+    uint32_t first;
+    uint32_t count;
+    bool grouped;
+};
+GM_HOST_DEVICE inline LaneShare lane_share(uint32_t chunk_count, uint32_t chunk_flags, uint32_t slice, uint32_t lane,
+                                           uint32_t vec, uint32_t block)
+{
+    LaneShare s{(slice * block + lane) * vec, 0u, false};
+    if (s.first >= chunk_count) return s;
+    const uint32_t vec_flag = vec == 4 ? kRecVec4Ok : kRecVec2Ok;
+    if (vec > 1 && (chunk_flags & vec_flag) != 0 && s.first + vec <= chunk_count) {
+        s.count = vec;
+        s.grouped = true;
+    } else {
+        const uint32_t left = chunk_count - s.first;
+        s.count = left < vec ? left : vec;
+    }
+    return s;
+}
+
 // log2(slices per chunk) for a chunk size, lane width and workgroup size; chunk_elements is a
 // power-of-two multiple of block * vec.
 uint32_t slice_shift_for(int chunk_elements, int vec, int block);

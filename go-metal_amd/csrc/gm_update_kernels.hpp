@@ -124,14 +124,12 @@ __device__ inline void update_slice(const Chunk &ch, uint32_t slice_shift, const
                                     float inv_scale)
 {
     const uint32_t slice = blockIdx.x & ((1u << slice_shift) - 1u);
-    const uint32_t local = (slice * BLOCK + threadIdx.x) * VEC;   // first element of this lane within the chunk
-    if (local >= ch.count) return;
-    constexpr uint32_t vec_flag = VEC == 4 ? kRecVec4Ok : kRecVec2Ok;
-    if (VEC > 1 && (ch.flags & vec_flag) && local + VEC <= ch.count) {
-        update_group<Rule, VEC, NT, AMP>(ch, local, prm, inv_scale);
+    const LaneShare s = lane_share(ch.count, ch.flags, slice, threadIdx.x, VEC, BLOCK);
+    if (s.count == 0) return;
+    if (VEC > 1 && s.grouped) {
+        update_group<Rule, VEC, NT, AMP>(ch, s.first, prm, inv_scale);
     } else {
-        const uint32_t n = ch.count - local < (uint32_t)VEC ? ch.count - local : (uint32_t)VEC;
-        for (uint32_t e = 0; e < n; e++) update_group<Rule, 1, NT, AMP>(ch, local + e, prm, inv_scale);
+        for (uint32_t e = 0; e < s.count; e++) update_group<Rule, 1, NT, AMP>(ch, s.first + e, prm, inv_scale);
     }
 }
 

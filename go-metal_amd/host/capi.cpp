@@ -307,8 +307,12 @@ try {
         fail(err);
         return nullptr;
     }
+    auto [js, jerr] = state->ToJSON();
+    if (!jerr.empty()) {
+        fail(jerr);
+        return nullptr;
+    }
     ok();
-    std::string js = state->ToJSON();
     char *out = (char *)std::malloc(js.size() + 1);
     if (out) std::memcpy(out, js.c_str(), js.size() + 1);
     return out;
@@ -336,8 +340,12 @@ try {
         fail(perr);
         return nullptr;
     }
+    auto [js, jerr] = state.ToJSON();
+    if (!jerr.empty()) {
+        fail(jerr);
+        return nullptr;
+    }
     ok();
-    std::string js = state.ToJSON();
     char *out = (char *)std::malloc(js.size() + 1);
     if (out) std::memcpy(out, js.c_str(), js.size() + 1);
     return out;
@@ -354,8 +362,12 @@ try {
         fail(err);
         return nullptr;
     }
+    auto [js, jerr] = state->ToCheckpointJSON();
+    if (!jerr.empty()) {
+        fail(jerr);
+        return nullptr;
+    }
     ok();
-    std::string js = state->ToCheckpointJSON();
     char *out = (char *)std::malloc(js.size() + 1);
     if (out) std::memcpy(out, js.c_str(), js.size() + 1);
     return out;

@@ -108,10 +108,27 @@ bool extractBoolParam(const std::map<std::string, ParamValue> &params, const std
     return defaultValue;
 }
 
+// Go's uint64(float64) of a value outside the target range is implementation-defined; in C++ it
+// is undefined behaviour.  Out-of-range counts saturate and NaN counts as zero.
+static uint64_t toUint64(double v)
+{
+    if (!(v >= 0.0)) return 0;                                   // negative or NaN
+    if (v >= 18446744073709551616.0) return UINT64_MAX;
+    return (uint64_t)v;
+}
+
+static int toInt(double v)
+{
+    if (std::isnan(v)) return 0;
+    if (v <= -2147483648.0) return INT32_MIN;
+    if (v >= 2147483647.0) return INT32_MAX;
+    return (int)v;
+}
+
 uint64_t extractUint64Param(const std::map<std::string, ParamValue> &params, const std::string &key,
                             uint64_t defaultValue)
 {
-    if (const double *v = asFloat64(params, key)) return (uint64_t)*v;
+    if (const double *v = asFloat64(params, key)) return toUint64(*v);
     return defaultValue;
 }
 
@@ -120,7 +137,7 @@ static void loadStepCountLenient(const std::map<std::string, ParamValue> &params
 {
     auto it = params.find("step_count");
     if (it == params.end()) return;
-    if (const double *d = std::get_if<double>(&it->second)) step = (uint64_t)*d;
+    if (const double *d = std::get_if<double>(&it->second)) step = toUint64(*d);
     else if (const uint64_t *u = std::get_if<uint64_t>(&it->second)) step = *u;
 }
 
@@ -546,13 +563,13 @@ Error AdamOptimizerState::LoadState(const OptimizerState *state)
     setFloat(state->Parameters, "beta2", Beta2);
     setFloat(state->Parameters, "epsilon", Epsilon);
     setFloat(state->Parameters, "weight_decay", WeightDecay);
-    if (const double *sc = asFloat64(state->Parameters, "step_count")) StepCount = (uint64_t)*sc;
+    if (const double *sc = asFloat64(state->Parameters, "step_count")) StepCount = toUint64(*sc);
     if (ampState) {
         const double *ls = asFloat64(state->Parameters, "loss_scale");
         const double *gt = asFloat64(state->Parameters, "growth_tracker");
         if (ls || gt) {
             if (ls) LossScale = (float)*ls;
-            if (gt) GrowthTracker = (int)*gt;
+            if (gt) GrowthTracker = toInt(*gt);
             if (gm_amp_state_set(reinterpret_cast<uintptr_t>(ampState), LossScale, GrowthTracker) != 0)
                 return Errorf("failed to restore loss-scale state: %s", gm_last_error());
         }
@@ -718,7 +735,7 @@ Error RMSPropOptimizerState::LoadState(const OptimizerState *state)
     setFloat(state->Parameters, "weight_decay", WeightDecay);
     setFloat(state->Parameters, "momentum", Momentum);
     Centered = extractBoolParam(state->Parameters, "centered", Centered);
-    if (const double *sc = asFloat64(state->Parameters, "step_count")) StepCount = (uint64_t)*sc;
+    if (const double *sc = asFloat64(state->Parameters, "step_count")) StepCount = toUint64(*sc);
     for (const OptimizerTensor &tensor : state->StateData) {
         int idx;
         if (Error e = checkTensor(tensor, bufferSizes, idx); !e.empty()) return e;

@@ -40,7 +40,8 @@ struct OptimizerState {
     std::vector<checkpoints::OptimizerTensor> StateData;
 
     // encoding/json shape: {"type":..,"parameters":{..},"state_data":[{"name","shape","data","state_type"}]}
-    std::string ToJSON() const;
+    // Fails on a non-finite value, as json.Marshal does ("json: unsupported value: NaN").
+    std::pair<std::string, Error> ToJSON() const;
     static std::pair<OptimizerState, Error> FromJSON(const std::string &text);
 
     // The reference stores this object under the key "optimizer_state" of its JSON checkpoint
@@ -49,7 +50,7 @@ struct OptimizerState {
     // checkpoint document that carries only the optimizer state and the metadata block
     // (framework "go-metal", version "1.0.0"), which the reference's loadJSON decodes.
     static std::pair<OptimizerState, Error> FromCheckpointJSON(const std::string &text);
-    std::string ToCheckpointJSON() const;
+    std::pair<std::string, Error> ToCheckpointJSON() const;
 };
 
 // optimizer/interface.go:13-43

@@ -37,10 +37,13 @@ static void appendEscaped(std::string &out, const std::string &s)
     out.push_back('"');
 }
 
-static void appendFloat(std::string &out, double v, int digits)
+// JSON has no inf / NaN: encoding/json's Marshal fails with an UnsupportedValueError
+// ("json: unsupported value: NaN"), and so does this encoder; `bad` receives Go's spelling of
+// the first such value.
+static void appendFloat(std::string &out, double v, int digits, std::string &bad)
 {
-    // JSON has no inf / NaN (encoding/json refuses them); they are written as null.
     if (!std::isfinite(v)) {
+        if (bad.empty()) bad = std::isnan(v) ? "NaN" : (v > 0 ? "+Inf" : "-Inf");
         out += "null";
         return;
     }
@@ -49,9 +52,9 @@ static void appendFloat(std::string &out, double v, int digits)
     out += buf;
 }
 
-std::string OptimizerState::ToJSON() const
+std::pair<std::string, Error> OptimizerState::ToJSON() const
 {
-    std::string out;
+    std::string out, bad;
     out.reserve(256 + StateData.size() * 64);
     out += "{\"type\":";
     appendEscaped(out, Type);
@@ -62,8 +65,8 @@ std::string OptimizerState::ToJSON() const
         first = false;
         appendEscaped(out, kv.first);
         out.push_back(':');
-        if (const double *d = std::get_if<double>(&kv.second)) appendFloat(out, *d, 17);
-        else if (const float *f = std::get_if<float>(&kv.second)) appendFloat(out, *f, 9);
+        if (const double *d = std::get_if<double>(&kv.second)) appendFloat(out, *d, 17, bad);
+        else if (const float *f = std::get_if<float>(&kv.second)) appendFloat(out, *f, 9, bad);
         else if (const bool *b = std::get_if<bool>(&kv.second)) out += *b ? "true" : "false";
         else if (const uint64_t *u = std::get_if<uint64_t>(&kv.second)) out += std::to_string(*u);
         else appendEscaped(out, std::get<std::string>(kv.second));
@@ -82,14 +85,15 @@ std::string OptimizerState::ToJSON() const
         out += "],\"data\":[";
         for (size_t i = 0; i < tensor.Data.size(); i++) {
             if (i) out.push_back(',');
-            appendFloat(out, tensor.Data[i], 9);
+            appendFloat(out, tensor.Data[i], 9, bad);
         }
         out += "],\"state_type\":";
         appendEscaped(out, tensor.StateType);
         out.push_back('}');
     }
     out += "]}";
-    return out;
+    if (!bad.empty()) return {std::string(), Errorf("json: unsupported value: %s", bad.c_str())};
+    return {std::move(out), ""};
 }
 
 namespace {
@@ -157,19 +161,40 @@ struct Parser {
         p++;
         return true;
     }
+    // A JSON number, by the JSON grammar only: -? (0 | [1-9][0-9]*) (. [0-9]+)? ([eE] [+-]? [0-9]+)?
+    // (strtod alone would also take "nan", "inf", hex floats and a leading '+').  A value beyond the
+    // float64 range is an error, as in encoding/json ("cannot unmarshal number 1e400").
     bool number(double &out)
     {
         ws();
-        if (end - p >= 4 && std::strncmp(p, "null", 4) == 0) {
-            p += 4;
-            out = std::nan("");
-            return true;
+        const char *q = p;
+        if (q < end && *q == '-') q++;
+        if (q >= end || *q < '0' || *q > '9') return fail("expected a number");
+        if (*q == '0') q++;
+        else while (q < end && *q >= '0' && *q <= '9') q++;
+        if (q < end && *q == '.') {
+            q++;
+            if (q >= end || *q < '0' || *q > '9') return fail("expected a digit after the decimal point");
+            while (q < end && *q >= '0' && *q <= '9') q++;
         }
-        char *stop = nullptr;
-        out = std::strtod(p, &stop);
-        if (stop == p) return fail("expected a number");
-        p = stop;
+        if (q < end && (*q == 'e' || *q == 'E')) {
+            q++;
+            if (q < end && (*q == '+' || *q == '-')) q++;
+            if (q >= end || *q < '0' || *q > '9') return fail("expected a digit in the exponent");
+            while (q < end && *q >= '0' && *q <= '9') q++;
+        }
+        const std::string token(p, q);           // strtod needs a terminated string of exactly this token
+        out = std::strtod(token.c_str(), nullptr);
+        if (!std::isfinite(out)) return fail("number out of range");
+        p = q;
         return true;
+    }
+    // An element of a []float32 / []int: a JSON null leaves the element at zero, as encoding/json
+    // does ("the JSON null value has no effect" on a non-pointer value).
+    bool elementIsNull()
+    {
+        ws();
+        return literal("null");
     }
     bool literal(const char *word)
     {
@@ -217,17 +242,19 @@ struct Parser {
 
 }  // namespace
 
-std::string OptimizerState::ToCheckpointJSON() const
+std::pair<std::string, Error> OptimizerState::ToCheckpointJSON() const
 {
     // field order of checkpoints.Checkpoint (checkpoint.go:38-52); a nil model spec and weight
     // list encode as null, the zero TrainingState as zeros
     std::string out = "{\"model_spec\":null,\"weights\":null,\"training_state\":{\"epoch\":0,\"step\":0,"
                       "\"learning_rate\":0,\"best_loss\":0,\"best_accuracy\":0,\"total_steps\":0},"
                       "\"optimizer_state\":";
-    out += ToJSON();
+    auto [body, err] = ToJSON();
+    if (!err.empty()) return {std::string(), err};
+    out += body;
     out += ",\"metadata\":{\"version\":\"1.0.0\",\"framework\":\"go-metal\","
            "\"created_at\":\"0001-01-01T00:00:00Z\"}}";
-    return out;
+    return {std::move(out), ""};
 }
 
 std::pair<OptimizerState, Error> OptimizerState::FromCheckpointJSON(const std::string &text)
@@ -284,6 +311,8 @@ std::pair<OptimizerState, Error> OptimizerState::FromJSON(const std::string &tex
                             st.Parameters[name] = false;
                         } else if (ps.peek('{') || ps.peek('[')) {
                             if (!ps.skip()) return {st, ps.err};
+                        } else if (ps.literal("null")) {
+                            // a nil interface value: every typed lookup falls back to its default
                         } else {
                             double d;
                             if (!ps.number(d)) return {st, ps.err};
@@ -323,10 +352,24 @@ std::pair<OptimizerState, Error> OptimizerState::FromJSON(const std::string &tex
                                             if (!ps.expect('[')) return {st, ps.err};
                                             if (!ps.peek(']')) {
                                                 for (;;) {
-                                                    double d;
-                                                    if (!ps.number(d)) return {st, ps.err};
-                                                    if (f == "shape") t.Shape.push_back((int)d);
-                                                    else t.Data.push_back((float)d);
+                                                    double d = 0;
+                                                    if (!ps.elementIsNull() && !ps.number(d)) return {st, ps.err};
+                                                    if (f == "shape") {
+                                                        // an int field: integral and in range, else
+                                                        // "cannot unmarshal number into Go struct field of type int"
+                                                        if (d != std::floor(d) || d < -2147483648.0 || d > 2147483647.0) {
+                                                            ps.fail("shape entry is not an int");
+                                                            return {st, ps.err};
+                                                        }
+                                                        t.Shape.push_back((int)d);
+                                                    } else {
+                                                        // a float32 field: a value that rounds to infinity is refused
+                                                        if (std::fabs(d) > 3.4028235677973366e38) {
+                                                            ps.fail("data entry is out of the float32 range");
+                                                            return {st, ps.err};
+                                                        }
+                                                        t.Data.push_back((float)d);
+                                                    }
                                                     if (ps.peek(',')) {
                                                         ps.p++;
                                                         continue;

@@ -9,6 +9,7 @@
  */
 #include "oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <string.h>
 
@@ -356,7 +357,8 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
 {
     const int nt = clamp_threads(nthreads);
     if (gm_oracle_amp_found_inf(g16, n, num_tensors, nthreads)) {
-        st->scale = st->scale * st->backoff_factor;
+        const float next = st->scale * st->backoff_factor;
+        if (next >= FLT_MIN) st->scale = next;        /* the scale stays a normal number */
         st->growth_tracker = 0;
         return 1;
     }
@@ -381,7 +383,8 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
     }
     st->growth_tracker += 1;
     if (st->growth_tracker == st->growth_interval) {
-        st->scale = st->scale * st->growth_factor;
+        const float next = st->scale * st->growth_factor;
+        if (next <= FLT_MAX) st->scale = next;        /* "up to maximum": never +inf */
         st->growth_tracker = 0;
     }
     return 0;

@@ -101,7 +101,10 @@ int gm_oracle_amp_found_inf(const uint16_t *const *g16, const size_t *n, int num
  * skipped (w, m, v, w16 and step_count untouched; scale *= backoff; tracker = 0),
  * else 0 (step_count++, g = float(g16) * (1.0f / scale), the Adam rule above,
  * w16 = half(w'), tracker++, and scale *= growth when tracker reaches the
- * interval). */
+ * interval).  The scale stays a normal finite number: a growth whose product exceeds
+ * FLT_MAX and a backoff whose product falls below FLT_MIN are not applied (the
+ * reference's tutorial: "scale = scale * 2 (up to maximum)",
+ * docs/tutorials/mixed-precision.md:624; it names no value). */
 int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *const *m,
                             float *const *v, uint16_t *const *w16, const size_t *n, int num_tensors,
                             float lr, float beta1, float beta2, float eps, float weight_decay,

@@ -385,6 +385,10 @@ def f16_bits_from_value(x: Fraction) -> int:
     return sign | ((e + 15) << 10) | man
 
 
+F32_OVERFLOW = Fraction(2 ** 128 - 2 ** 103)      # values from here up round to +inf (ties to even)
+F32_MIN_NORMAL = Fraction(1, 2 ** 126)
+
+
 def run_amp_case(name, hp, amp, w0, g16_steps):
     """g16_steps: list of steps; each step is a list of tensors; each tensor a list of half bits."""
     h = derive("adam", hp)
@@ -402,7 +406,8 @@ def run_amp_case(name, hp, amp, w0, g16_steps):
     for g16 in g16_steps:
         found = any(f16_value(b) is None for t in g16 for b in t)
         if found:
-            scale = rf32(scale * backoff)
+            if rf32(scale * backoff) >= F32_MIN_NORMAL:      # the scale stays a normal, finite number
+                scale = rf32(scale * backoff)
             tracker = 0
         else:
             step_count += 1
@@ -415,7 +420,8 @@ def run_amp_case(name, hp, amp, w0, g16_steps):
                     w16[ti][i] = f16_bits_from_value(w[ti][i])
             tracker += 1
             if tracker == interval:
-                scale = rf32(scale * growth)
+                if scale * growth < F32_OVERFLOW:                # the product rounds to a finite binary32
+                    scale = rf32(scale * growth)
                 tracker = 0
         trace.append({
             "skipped": int(found), "scale": f32_bits(scale), "growth_tracker": tracker,

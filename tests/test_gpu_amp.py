@@ -308,3 +308,34 @@ def test_random_lists_scales_and_injections(dev, seed):
         pair.compare(f"seed {seed}")
     finally:
         pair.close()
+
+
+def test_loss_scale_stays_finite_and_normal(dev):
+    """Gradients that never overflow make the scale grow at every interval; it must stop at the largest
+    finite power of two (not +inf, where inf * 0.5 = inf would hold it for good and 1 / scale = 0 would
+    zero every gradient), and a run of overflows must stop at the smallest normal number.  Device state
+    machine against the oracle's, every step."""
+    w0 = [np.linspace(-0.5, 0.5, 300).astype(np.float32), np.full(5, 0.25, np.float32)]
+    pair = AmpPair(dev, w0, HYPER, (2.0 ** 125, 2.0, 0.5, 1))
+    try:
+        zero = [np.zeros(s, np.uint16) for s in pair.sizes]
+        scales = []
+        for _ in range(5):
+            assert pair.step(zero) == 0
+            scales.append(float(pair.st.scale))
+        assert scales == [2.0 ** 126] + [2.0 ** 127] * 4
+        pair.compare("scale at its ceiling")
+    finally:
+        pair.close()
+    pair = AmpPair(dev, w0, HYPER, (2.0 ** -124, 2.0, 0.5, 1000))
+    try:
+        bad = [np.zeros(s, np.uint16) for s in pair.sizes]
+        bad[1][4] = 0xFC00
+        scales = []
+        for _ in range(5):
+            assert pair.step(bad) == 1
+            scales.append(float(pair.st.scale))
+        assert scales == [2.0 ** -125] + [2.0 ** -126] * 4
+        pair.compare("scale at its floor")
+    finally:
+        pair.close()

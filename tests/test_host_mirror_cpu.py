@@ -246,8 +246,8 @@ def test_optimizer_state_json_shape_and_field_handling():
     assert err is None and json.loads(out) == {"type": "RMSProp", "parameters": {}, "state_data": []}
     out, err = normalize('{"type":"Adam","parameters":{},"state_data":[{"name":"v_1","shape":[2],'
                          '"data":[1.5,null],"state_type":"variance"}]}')
-    assert err is None                                      # null decodes to NaN and is written back as null
-    assert json.loads(out)["state_data"][0]["data"] == [1.5, None]
+    assert err is None                                      # "the JSON null value has no effect": the element stays 0
+    assert json.loads(out)["state_data"][0]["data"] == [1.5, 0]
     out, err = normalize('{"type":"A","state_data":[{"name":"x","shape":[1],"data":[1],"state_type":"s"}],'
                          '"type":"B","state_data":[]}')
     assert err is None and json.loads(out) == {"type": "B", "parameters": {}, "state_data": []}   # last key wins
@@ -255,6 +255,34 @@ def test_optimizer_state_json_shape_and_field_handling():
                    '{"type":"Adam"} trailing'):
         out, err = normalize(broken)
         assert out is None and err.startswith("invalid optimizer state JSON"), (broken, out, err)
+
+
+def test_optimizer_state_json_numbers_follow_the_json_grammar():
+    """Numbers are JSON numbers and nothing else: what strtod would also take (nan, inf, hex, a leading
+    plus, a bare leading or trailing point) is refused, and so are values beyond the target type's
+    range, as in encoding/json ("cannot unmarshal number 1e400 into Go value of type float64",
+    "... number 1e39 into Go struct field .data of type float32", "... number 1.5 into ... of type int")."""
+    param = '{"type":"Adam","parameters":{"a":%s},"state_data":[]}'
+    for good in ("0", "-0", "12", "-1.5", "1e5", "1E-5", "0.5e+3", "1.7976931348623157e308", "4.9e-324"):
+        out, err = normalize(param % good)
+        assert err is None, (good, err)
+    for bad in ("nan", "NaN", "-inf", "inf", "Infinity", "0x10", "+1", "01", "1.", ".5", "1e", "1e+", "--1", "1e400",
+                "-1e400"):
+        out, err = normalize(param % bad)
+        assert out is None and err.startswith("invalid optimizer state JSON"), (bad, out)
+    tensor = '{"type":"Adam","parameters":{},"state_data":[{"name":"m_0","shape":[%s],"data":[%s],"state_type":"m"}]}'
+    for shape, data, ok in (("2", "1,2", True), ("2", "3.4028234e38,-3.4028234e38", True), ("1", "1e39", False),
+                            ("1", "-1e39", False), ("1", "3.5e38", False), ("1.5", "1", False), ("1e10", "1", False),
+                            ("-3", "1", True), ("null", "null", True)):
+        out, err = normalize(tensor % (shape, data))
+        assert (err is None) == ok, (shape, data, err)
+    # a parameter of null is a nil interface value: present in no typed lookup, absent after re-encoding
+    out, err = normalize(param % "null")
+    assert err is None and json.loads(out)["parameters"] == {}
+    # counts outside the uint64 range saturate (Go leaves the conversion implementation-defined)
+    assert lib.gmo_extract_uint64_param(b'{"step_count":-5}', b"step_count", 7) == 0
+    assert lib.gmo_extract_uint64_param(b'{"step_count":1e300}', b"step_count", 7) == 2 ** 64 - 1
+    assert lib.gmo_extract_uint64_param(b'{"step_count":41}', b"step_count", 7) == 41
 
 
 # ---- memory.Tensor helpers

@@ -200,13 +200,16 @@ def amp_reference_sequence(flags, init_scale, growth, backoff, interval):
     """Brute-force state machine in pure Python over a list of overflow flags."""
     scale, tracker, steps, out = np.float32(init_scale), 0, 0, []
     for f in flags:
-        if f:
-            scale, tracker = np.float32(scale * np.float32(backoff)), 0
-        else:
-            steps += 1
-            tracker += 1
-            if tracker == interval:
-                scale, tracker = np.float32(scale * np.float32(growth)), 0
+        with np.errstate(over="ignore", under="ignore"):
+            if f:
+                lower = np.float32(scale * np.float32(backoff))
+                scale, tracker = (lower if lower >= np.finfo(np.float32).tiny else scale), 0
+            else:
+                steps += 1
+                tracker += 1
+                if tracker == interval:
+                    higher = np.float32(scale * np.float32(growth))
+                    scale, tracker = (higher if np.isfinite(higher) else scale), 0
         out.append((int(f), float(scale), tracker, steps))
     return out
 
@@ -238,3 +241,30 @@ def test_amp_skip_and_scale_sequence_against_brute_force():
         else:
             for a, h in zip(w, w16):
                 assert np.array_equal(h, a.astype(np.float16).view(np.uint16))
+
+
+def test_amp_scale_stays_finite_and_normal():
+    """Zero gradients never overflow, so the scale grows at every interval: it must stop at the largest
+    finite power of two instead of reaching +inf (where inf * backoff = inf would hold it for good), and
+    a run of overflows must stop at the smallest normal number instead of reaching zero.
+    Perturbation tried: the two range checks removed from oracle.c -> this test fails at step 3 / 4."""
+    o = oracle()
+    n = [8]
+    w, m, v, w16 = [rand(0.1, 8)], [np.zeros(8, np.float32)], [np.zeros(8, np.float32)], [np.zeros(8, np.uint16)]
+    st = o.amp_state(2.0 ** 125, 2.0, 0.5, 1)
+    zero = [np.zeros(8, np.uint16)]
+    scales = []
+    for _ in range(5):
+        assert o.adam_amp(w, zero, m, v, w16, 1e-3, 0.9, 0.999, 1e-8, 0.0, st) == 0
+        scales.append(float(st.scale))
+    assert scales == [2.0 ** 126, 2.0 ** 127, 2.0 ** 127, 2.0 ** 127, 2.0 ** 127]
+    assert [s for _, s, _, _ in amp_reference_sequence([0] * 5, 2.0 ** 125, 2.0, 0.5, 1)] == scales
+    assert np.all(np.isfinite(w[0]))
+    st = o.amp_state(2.0 ** -124, 2.0, 0.5, 1000)
+    bad = [np.full(8, 0x7C00, np.uint16)]
+    scales = []
+    for _ in range(5):
+        assert o.adam_amp(w, bad, m, v, w16, 1e-3, 0.9, 0.999, 1e-8, 0.0, st) == 1
+        scales.append(float(st.scale))
+    assert scales == [2.0 ** -125, 2.0 ** -126, 2.0 ** -126, 2.0 ** -126, 2.0 ** -126]
+    assert [s for _, s, _, _ in amp_reference_sequence([1] * 5, 2.0 ** -124, 2.0, 0.5, 1000)] == scales
