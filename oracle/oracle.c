@@ -318,18 +318,68 @@ float gm_oracle_f16_to_f32(uint16_t h)
     return f;
 }
 
+/* The two conversions above are the reference: one branch per class of value.  The loops
+ * below run them over hundreds of millions of elements per step, so the common class (a result
+ * in the normal half range) is handled inline by integer arithmetic and everything else falls
+ * through to the reference.  gm_oracle_f16_fast_mismatches compares the two forms over any
+ * range of bit patterns; the tests run it over all 2^32 floats and all 2^16 halves. */
+static inline float f16_to_f32_fast(uint16_t h)
+{
+    const uint32_t em = (uint32_t)h & 0x7FFFu;
+    if (em - 0x0400u < 0x7800u) {               /* exponent field 1..30: a normal half */
+        const uint32_t u = (((uint32_t)h & 0x8000u) << 16) | ((em << 13) + 0x38000000u);
+        float f;
+        memcpy(&f, &u, sizeof f);
+        return f;
+    }
+    return gm_oracle_f16_to_f32(h);
+}
+
+static inline uint16_t f32_to_f16_fast(float x)
+{
+    uint32_t u;
+    memcpy(&u, &x, sizeof u);
+    const uint32_t a = u & 0x7FFFFFFFu;
+    /* 2^-14 <= |x| < 65504: the result is a normal half and rounding cannot reach infinity */
+    if (a - 0x38800000u < 0x477FE000u - 0x38800000u) {
+        const uint32_t r = a + 0xFFFu + ((a >> 13) & 1u);     /* nearest, ties to even, at bit 13 */
+        return (uint16_t)(((u >> 16) & 0x8000u) | ((r - 0x38000000u) >> 13));
+    }
+    return gm_oracle_f32_to_f16(x);
+}
+
+uint64_t gm_oracle_f16_fast_mismatches(uint64_t first_bits, uint64_t count, int halves, int nthreads)
+{
+    const int nt = clamp_threads(nthreads);
+    uint64_t bad = 0;
+    #pragma omp parallel for schedule(static) num_threads(nt) if(nt > 1) reduction(+:bad)
+    for (uint64_t k = 0; k < count; k++) {
+        if (halves) {
+            const uint16_t h = (uint16_t)(first_bits + k);
+            const float a = f16_to_f32_fast(h), b = gm_oracle_f16_to_f32(h);
+            bad += memcmp(&a, &b, sizeof a) != 0;
+        } else {
+            const uint32_t u = (uint32_t)(first_bits + k);
+            float x;
+            memcpy(&x, &u, sizeof x);
+            bad += f32_to_f16_fast(x) != gm_oracle_f32_to_f16(x);
+        }
+    }
+    return bad;
+}
+
 void gm_oracle_convert_f32_to_f16(const float *src, uint16_t *dst, size_t n, int nthreads)
 {
     const int nt = clamp_threads(nthreads);
     GM_PARALLEL_FOR
-    for (size_t i = 0; i < n; i++) dst[i] = gm_oracle_f32_to_f16(src[i]);
+    for (size_t i = 0; i < n; i++) dst[i] = f32_to_f16_fast(src[i]);
 }
 
 void gm_oracle_convert_f16_to_f32(const uint16_t *src, float *dst, size_t n, int nthreads)
 {
     const int nt = clamp_threads(nthreads);
     GM_PARALLEL_FOR
-    for (size_t i = 0; i < n; i++) dst[i] = gm_oracle_f16_to_f32(src[i]);
+    for (size_t i = 0; i < n; i++) dst[i] = f16_to_f32_fast(src[i]);
 }
 
 /* ---- mixed-precision Adam ---- */
@@ -375,10 +425,10 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
         const size_t cnt = n[t];
         GM_PARALLEL_FOR
         for (size_t i = 0; i < cnt; i++) {
-            float gi = gm_oracle_f16_to_f32(gt[i]) * inv_scale;
+            float gi = f16_to_f32_fast(gt[i]) * inv_scale;
             adam_element(&wt[i], gi, &mt[i], &vt[i], lr, beta1, beta2, omb1, omb2,
                          eps, weight_decay, bc1, bc2);
-            ht[i] = gm_oracle_f32_to_f16(wt[i]);
+            ht[i] = f32_to_f16_fast(wt[i]);
         }
     }
     st->growth_tracker += 1;

@@ -80,6 +80,10 @@ void gm_oracle_nadam_step(float *w, const float *g, float *m, float *v, size_t n
  * hardware conversion instruction. */
 uint16_t gm_oracle_f32_to_f16(float x);
 float    gm_oracle_f16_to_f32(uint16_t h);
+/* Number of bit patterns in [first_bits, first_bits + count) on which the inlined fast forms of
+ * the two conversions (used by the bulk loops) differ from the functions above: fp32 patterns
+ * through f32 -> f16, or (halves != 0) fp16 patterns through f16 -> f32.  Must be 0. */
+uint64_t gm_oracle_f16_fast_mismatches(uint64_t first_bits, uint64_t count, int halves, int nthreads);
 void gm_oracle_convert_f32_to_f16(const float *src, uint16_t *dst, size_t n, int nthreads);
 void gm_oracle_convert_f16_to_f32(const uint16_t *src, float *dst, size_t n, int nthreads);
 

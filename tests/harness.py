@@ -32,6 +32,19 @@ def states_for(rule, hyper):
     return STATE_NAMES[rule]
 
 
+def progress(message):
+    """A line for whoever watches a long GPU test from outside: pytest captures stdout, so the line also goes
+    to a file the GPU job's output folder carries back (and that marks the job as alive)."""
+    print(message, flush=True)
+    try:
+        folder = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(folder, exist_ok=True)
+        with open(os.path.join(folder, "test_progress.log"), "a") as f:
+            f.write(message + "\n")
+    except OSError:
+        pass
+
+
 _GPU = None
 
 

@@ -1,0 +1,173 @@
+"""The mixed-precision configurations at their stated size and length.
+
+config 4: 125,000,000 parameters in 60 tensors, 5000 steps, fp16 gradients N(0, 1e-4) x the current loss
+scale regenerated on the device for every step, +inf / -inf / NaN written into one random element on a
+seeded 0.5 % of steps, loss scale 65536 with backoff x0.5 and growth x2 every 2000 clean steps.
+config 5 (mixed-precision variant): 1,012,301,824 parameters in 400 tensors, weight decay 1e-4, 20 steps.
+
+Every step's (skipped, scale, clean-step counter, step count) must equal the CPU oracle's, and weights,
+moments and the fp16 weight copy are compared bit for bit at checkpoints (every 500 steps / steps 1, 10, 20).
+The oracle consumes the very gradients the device generated (read back once per step) and runs in a worker
+thread one step behind the GPU, so the run takes about as long as the oracle alone."""
+import ctypes
+import os
+import queue
+import threading
+import time
+
+import numpy as np
+import pytest
+
+from harness import gpu_device, progress
+from oracle_lib import oracle
+from workloads import amp_125m_sizes, transformer_block_sizes
+from __graft_entry__ import load_package
+
+pytestmark = pytest.mark.gpu
+NTHREADS = min(16, os.cpu_count() or 1)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = gpu_device()
+    if d is None:
+        pytest.fail("libgometal_hip.so is missing or no GPU is usable: GPU tests cannot run")
+    return d
+
+
+def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
+    """inject_at: {step index: (tensor, element, fp16 bits)}; checkpoints: step indices (0-based) after which
+    all buffers are compared."""
+    pkg, lib, D, o = load_package(), dev.lib, dev.handle, oracle()
+    n, total = len(sizes), sum(sizes)
+    offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    rng = np.random.default_rng(seed)
+
+    # ---- device side: one parent buffer per fp16 stream, one buffer per tensor for the fp32 streams
+    w_host = [rng.standard_normal(s, dtype=np.float32) * np.float32(0.02) for s in sizes]
+    d_w = [dev.from_numpy(a) for a in w_host]
+    d_m = [dev.alloc(4 * s, zero=True) for s in sizes]
+    d_v = [dev.alloc(4 * s, zero=True) for s in sizes]
+    d_g16 = dev.alloc(2 * total)
+    d_w16 = dev.alloc(2 * total, zero=True)
+    arr = pkg.handle_array
+    c_w, c_m, c_v = arr(d_w), arr(d_m), arr(d_v)
+    c_g16 = arr([d_g16 + 2 * int(off) for off in offsets[:-1]])
+    c_w16 = arr([d_w16 + 2 * int(off) for off in offsets[:-1]])
+    bs = pkg.int_array([4 * s for s in sizes])
+    amp = lib.gm_amp_state_create(D, 65536.0, 2.0, 0.5, 2000)
+    assert amp
+
+    # ---- oracle side
+    m_host = [np.zeros(s, np.float32) for s in sizes]
+    v_host = [np.zeros(s, np.float32) for s in sizes]
+    w16_host = [np.zeros(s, np.uint16) for s in sizes]
+    st = o.amp_state(65536.0, 2.0, 0.5, 2000)
+    g_buffers = [np.empty((2 * total + 3) // 4, np.uint32) for _ in range(2)]
+    free_buffers, work = queue.Queue(), queue.Queue(maxsize=1)
+    for b in range(2):
+        free_buffers.put(b)
+    oracle_trace, failure = [], []
+
+    def oracle_worker():
+        try:
+            while True:
+                item = work.get()
+                if item is None:
+                    return
+                b = item
+                g = g_buffers[b].view(np.uint16)
+                g16 = [g[offsets[k]:offsets[k + 1]] for k in range(n)]
+                skipped = o.adam_amp(w_host, g16, m_host, v_host, w16_host, state=st, nthreads=NTHREADS, **hyper)
+                oracle_trace.append((skipped, float(np.float32(st.scale)), st.growth_tracker, int(st.step_count)))
+                free_buffers.put(b)
+        except Exception as e:  # noqa: BLE001
+            failure.append(e)
+            free_buffers.put(-1)
+
+    worker = threading.Thread(target=oracle_worker, daemon=True)
+    worker.start()
+
+    def drain():
+        """Waits until the oracle has applied every step handed to it."""
+        held = [free_buffers.get(), free_buffers.get()]
+        assert not failure, failure
+        for b in held:
+            free_buffers.put(b)
+
+    def compare(context):
+        drain()
+        for name_, dh, host in (("w", d_w, w_host), ("m", d_m, m_host), ("v", d_v, v_host)):
+            for k in range(n):
+                got = dev.to_numpy(dh[k], sizes[k])
+                assert np.array_equal(got.view(np.uint32), host[k].view(np.uint32)), (context, name_, k)
+        got16 = dev.to_numpy(d_w16, total, np.uint16)
+        for k in range(n):
+            assert np.array_equal(got16[offsets[k]:offsets[k + 1]], w16_host[k]), (context, "w16", k)
+
+    gpu_trace = []
+    scale, applied = 65536.0, 0
+    t0 = time.time()
+    try:
+        for k in range(steps):
+            # this step's gradients at the current loss scale, made on the device
+            assert lib.gm_fill_normal_f16(D, d_g16, total, 0xC4000000 + 7919 * k + seed, 0.0, 1e-4, scale) == 0
+            if k in inject_at:
+                t, e, bits = inject_at[k]
+                tmp = dev.from_numpy(np.array([bits, 0], np.uint16))
+                assert lib.copy_buffer_to_buffer_sync(tmp, d_g16, 0, 2 * (int(offsets[t]) + e), 2) == 0
+                dev.free(tmp)
+            b = free_buffers.get()
+            assert b >= 0 and not failure, failure
+            words = g_buffers[b].size
+            assert lib.copy_metal_buffer_to_int32_array(d_g16, g_buffers[b].ctypes.data_as(ctypes.c_void_p), words) == 0
+            skipped, sc, tracker = ctypes.c_int(-1), ctypes.c_float(0), ctypes.c_int(-1)
+            rc = lib.execute_adam_amp_step(D, c_w, c_g16, c_m, c_v, c_w16, n, bs, hyper["lr"], hyper["beta1"],
+                                           hyper["beta2"], hyper["eps"], hyper["weight_decay"], applied + 1, amp,
+                                           ctypes.byref(skipped), ctypes.byref(sc), ctypes.byref(tracker))
+            assert rc == 0, (rc, lib.gm_last_error())
+            applied += 0 if skipped.value else 1
+            scale = sc.value
+            gpu_trace.append((skipped.value, sc.value, tracker.value, applied))
+            work.put(b)
+            if k % 50 == 0:
+                progress(f"{name}: step {k + 1} of {steps}, scale {scale}, {time.time() - t0:.0f} s")
+            if k in checkpoints:
+                compare(f"{name} after step {k + 1}")
+                assert gpu_trace == oracle_trace, next((i, a, b_) for i, (a, b_) in enumerate(zip(gpu_trace, oracle_trace)) if a != b_)
+        drain()
+        assert len(oracle_trace) == steps and gpu_trace == oracle_trace
+        want_skips = sorted(inject_at)
+        assert [i for i, t in enumerate(gpu_trace) if t[0]] == want_skips
+        return gpu_trace
+    finally:
+        work.put(None)
+        worker.join(timeout=60)
+        lib.gm_amp_state_destroy(amp)
+        for h in d_w + d_m + d_v + [d_g16, d_w16]:
+            dev.free(h)
+
+
+def test_config4_full_size_5000_steps(dev):
+    sizes = amp_125m_sizes()
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)
+    rng = np.random.default_rng(0x6D657461 + 4)
+    chosen = np.flatnonzero(rng.random(5000) < 0.005)
+    inject = {}
+    for j, k in enumerate(chosen):
+        t = int(rng.integers(0, len(sizes)))
+        inject[int(k)] = (t, int(rng.integers(0, sizes[t])), [0x7C00, 0xFC00, 0x7E00][j % 3])
+    assert len(inject) > 10
+    trace = run_schedule(dev, "config 4", sizes, hyper, 5000, inject, {499 + 500 * i for i in range(10)}, seed=4)
+    # the schedule really exercised both directions of the scale
+    scales = {t[1] for t in trace}
+    assert len(scales) >= 4 and min(scales) < 65536.0
+    assert trace[-1][3] == 5000 - len(inject)
+
+
+def test_config5_mixed_precision_full_size_20_steps(dev):
+    sizes = transformer_block_sizes()
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)
+    inject = {6: (len(sizes) - 3, 1234, 0xFC00), 13: (2, 4096 * 11008 - 1, 0x7E00)}
+    trace = run_schedule(dev, "config 5 mixed precision", sizes, hyper, 20, inject, {0, 9, 19}, seed=5)
+    assert [t[0] for t in trace].count(1) == 2 and trace[-1][1] == 16384.0 and trace[-1][3] == 18
