@@ -400,6 +400,121 @@ int gm_oracle_amp_found_inf(const uint16_t *const *g16, const size_t *n, int num
     return found;
 }
 
+/* Eight elements of the mixed-precision Adam step at once, for hosts with AVX2 and F16C: the
+ * same operations in the same order as the scalar loop below, each one a single IEEE
+ * binary32 operation per lane (explicit intrinsics, no FMA in the target set), the two
+ * conversions by the hardware (vcvtph2ps is exact, vcvtps2ph rounds to nearest even and
+ * quiets NaNs exactly like gm_oracle_f32_to_f16).  gm_oracle_amp_vector_mismatches runs both
+ * forms over the same data; the tests hold them to identical bits. */
+#if defined(__x86_64__)
+#include <immintrin.h>
+#define GM_HAVE_AMP_VECTOR 1
+__attribute__((target("avx2,f16c")))
+static void adam_amp_span_avx2(float *w, const uint16_t *g16, float *m, float *v, uint16_t *w16, size_t n,
+                               float lr, float beta1, float beta2, float omb1, float omb2, float eps,
+                               float weight_decay, float bc1, float bc2, float inv_scale)
+{
+    const __m256 vlr = _mm256_set1_ps(lr), vb1 = _mm256_set1_ps(beta1), vb2 = _mm256_set1_ps(beta2);
+    const __m256 vomb1 = _mm256_set1_ps(omb1), vomb2 = _mm256_set1_ps(omb2), veps = _mm256_set1_ps(eps);
+    const __m256 vwd = _mm256_set1_ps(weight_decay), vbc1 = _mm256_set1_ps(bc1), vbc2 = _mm256_set1_ps(bc2);
+    const __m256 vinv = _mm256_set1_ps(inv_scale);
+    const int decay_on = weight_decay > 0.0f;
+    for (size_t i = 0; i + 8 <= n; i += 8) {
+        const __m256 g = _mm256_mul_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(g16 + i))), vinv);
+        const __m256 wi = _mm256_loadu_ps(w + i);
+        const __m256 mi = _mm256_add_ps(_mm256_mul_ps(_mm256_loadu_ps(m + i), vb1), _mm256_mul_ps(g, vomb1));
+        const __m256 vi = _mm256_add_ps(_mm256_mul_ps(_mm256_loadu_ps(v + i), vb2),
+                                        _mm256_mul_ps(_mm256_mul_ps(g, g), vomb2));
+        const __m256 m_hat = _mm256_div_ps(mi, vbc1);
+        const __m256 v_hat = _mm256_div_ps(vi, vbc2);
+        const __m256 den = _mm256_add_ps(_mm256_sqrt_ps(v_hat), veps);
+        __m256 upd = _mm256_div_ps(m_hat, den);
+        if (decay_on) upd = _mm256_add_ps(upd, _mm256_mul_ps(wi, vwd));
+        const __m256 wn = _mm256_sub_ps(wi, _mm256_mul_ps(upd, vlr));
+        _mm256_storeu_ps(w + i, wn);
+        _mm256_storeu_ps(m + i, mi);
+        _mm256_storeu_ps(v + i, vi);
+        _mm_storeu_si128((__m128i *)(w16 + i), _mm256_cvtps_ph(wn, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC));
+    }
+}
+static int amp_vector_usable(void)
+{
+    return __builtin_cpu_supports("avx2") && __builtin_cpu_supports("f16c");
+}
+#else
+#define GM_HAVE_AMP_VECTOR 0
+#endif
+
+/* One tensor of the applied step: elements [0, n).  use_vector = 0 forces the scalar form. */
+static void adam_amp_tensor(float *wt, const uint16_t *gt, float *mt, float *vt, uint16_t *ht, size_t cnt,
+                            float lr, float beta1, float beta2, float omb1, float omb2, float eps,
+                            float weight_decay, float bc1, float bc2, float inv_scale, int nt, int use_vector)
+{
+#if GM_HAVE_AMP_VECTOR
+    if (use_vector && amp_vector_usable()) {
+        /* spans of a multiple of eight elements per thread; the tail below is scalar */
+        const size_t span = 1u << 16;
+        const size_t spans = cnt / span;
+        #pragma omp parallel for schedule(static) num_threads(nt) if(nt > 1)
+        for (size_t s = 0; s < spans; s++)
+            adam_amp_span_avx2(wt + s * span, gt + s * span, mt + s * span, vt + s * span, ht + s * span, span, lr,
+                               beta1, beta2, omb1, omb2, eps, weight_decay, bc1, bc2, inv_scale);
+        const size_t done = spans * span;
+        const size_t rest8 = (cnt - done) / 8 * 8;
+        adam_amp_span_avx2(wt + done, gt + done, mt + done, vt + done, ht + done, rest8, lr, beta1, beta2, omb1,
+                           omb2, eps, weight_decay, bc1, bc2, inv_scale);
+        wt += done + rest8, gt += done + rest8, mt += done + rest8, vt += done + rest8, ht += done + rest8;
+        cnt -= done + rest8;
+    }
+#else
+    (void)use_vector;
+#endif
+    GM_PARALLEL_FOR
+    for (size_t i = 0; i < cnt; i++) {
+        float gi = f16_to_f32_fast(gt[i]) * inv_scale;
+        adam_element(&wt[i], gi, &mt[i], &vt[i], lr, beta1, beta2, omb1, omb2,
+                     eps, weight_decay, bc1, bc2);
+        ht[i] = f32_to_f16_fast(wt[i]);
+    }
+}
+
+uint64_t gm_oracle_amp_vector_mismatches(const float *w, const uint16_t *g16, const float *m, const float *v,
+                                         size_t n, float lr, float beta1, float beta2, float eps,
+                                         float weight_decay, float bc1, float bc2, float inv_scale)
+{
+#if GM_HAVE_AMP_VECTOR
+    if (!amp_vector_usable()) return UINT64_MAX;
+    uint64_t bad = 0;
+    const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2;
+    float a[4][64], b[4][64];             /* w, m, v and (as floats) nothing: blocks of 64 elements */
+    uint16_t ha[64], hb[64];
+    for (size_t i = 0; i < n; i += 64) {
+        const size_t k = n - i < 64 ? n - i : 64;
+        memcpy(a[0], w + i, k * 4), memcpy(a[1], m + i, k * 4), memcpy(a[2], v + i, k * 4);
+        memcpy(b[0], w + i, k * 4), memcpy(b[1], m + i, k * 4), memcpy(b[2], v + i, k * 4);
+        memset(ha, 0, sizeof ha), memset(hb, 0, sizeof hb);
+        adam_amp_tensor(a[0], g16 + i, a[1], a[2], ha, k, lr, beta1, beta2, omb1, omb2, eps, weight_decay, bc1, bc2,
+                        inv_scale, 1, 1);
+        adam_amp_tensor(b[0], g16 + i, b[1], b[2], hb, k, lr, beta1, beta2, omb1, omb2, eps, weight_decay, bc1, bc2,
+                        inv_scale, 1, 0);
+        /* identical bits, except that any NaN equals any NaN: which operand's payload survives an
+         * operation on two NaNs depends on operand order, which the compiler is free to choose */
+        int differs = 0;
+        for (int q = 0; q < 3; q++)
+            for (size_t e = 0; e < k; e++)
+                differs |= memcmp(&a[q][e], &b[q][e], 4) != 0 && !(isnan(a[q][e]) && isnan(b[q][e]));
+        for (size_t e = 0; e < k; e++)
+            differs |= ha[e] != hb[e] && !((ha[e] & 0x7FFFu) > 0x7C00u && (hb[e] & 0x7FFFu) > 0x7C00u);
+        bad += differs;
+    }
+    return bad;
+#else
+    (void)w, (void)g16, (void)m, (void)v, (void)n, (void)lr, (void)beta1, (void)beta2, (void)eps;
+    (void)weight_decay, (void)bc1, (void)bc2, (void)inv_scale;
+    return UINT64_MAX;
+#endif
+}
+
 int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *const *m,
                             float *const *v, uint16_t *const *w16, const size_t *n, int num_tensors,
                             float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -418,19 +533,9 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
     const float omb1 = 1.0f - beta1;
     const float omb2 = 1.0f - beta2;
     const float inv_scale = 1.0f / st->scale;
-    for (int t = 0; t < num_tensors; t++) {
-        float *wt = w[t], *mt = m[t], *vt = v[t];
-        const uint16_t *gt = g16[t];
-        uint16_t *ht = w16[t];
-        const size_t cnt = n[t];
-        GM_PARALLEL_FOR
-        for (size_t i = 0; i < cnt; i++) {
-            float gi = f16_to_f32_fast(gt[i]) * inv_scale;
-            adam_element(&wt[i], gi, &mt[i], &vt[i], lr, beta1, beta2, omb1, omb2,
-                         eps, weight_decay, bc1, bc2);
-            ht[i] = f32_to_f16_fast(wt[i]);
-        }
-    }
+    for (int t = 0; t < num_tensors; t++)
+        adam_amp_tensor(w[t], g16[t], m[t], v[t], w16[t], n[t], lr, beta1, beta2, omb1, omb2, eps, weight_decay,
+                        bc1, bc2, inv_scale, nt, 1);
     st->growth_tracker += 1;
     if (st->growth_tracker == st->growth_interval) {
         const float next = st->scale * st->growth_factor;

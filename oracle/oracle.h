@@ -114,6 +114,14 @@ int gm_oracle_adam_amp_step(float *const *w, const uint16_t *const *g16, float *
                             float lr, float beta1, float beta2, float eps, float weight_decay,
                             gm_oracle_amp_state *st, int nthreads);
 
+/* The applied mixed-precision step has an eight-lane form for hosts with AVX2 and F16C (same
+ * operations, one IEEE operation per lane each).  This runs both forms over n elements in
+ * blocks of 64 and returns the number of blocks whose w / m / v / w16 differ in any bit, any
+ * NaN counting as equal to any NaN (must be 0); UINT64_MAX when the host cannot run the vector form. */
+uint64_t gm_oracle_amp_vector_mismatches(const float *w, const uint16_t *g16, const float *m, const float *v,
+                                         size_t n, float lr, float beta1, float beta2, float eps,
+                                         float weight_decay, float bc1, float bc2, float inv_scale);
+
 /* L-BFGS step, cgo_bridge/bridge_optimizer.m:980-1321 (oracle_lbfgs.c states what is
  * reproduced).  s and y hold history_size * num_tensors tensors, entry [h * num_tensors + i];
  * rho and alpha are host arrays of history_size floats (the reference keeps each rho in a

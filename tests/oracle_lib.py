@@ -67,6 +67,8 @@ class Oracle:
         L.gm_oracle_f16_to_f32.restype = f
         L.gm_oracle_f16_fast_mismatches.argtypes = [ctypes.c_uint64, ctypes.c_uint64, i, i]
         L.gm_oracle_f16_fast_mismatches.restype = ctypes.c_uint64
+        L.gm_oracle_amp_vector_mismatches.argtypes = [c_float_p, c_u16_p, c_float_p, c_float_p, sz] + [f] * 8
+        L.gm_oracle_amp_vector_mismatches.restype = ctypes.c_uint64
         L.gm_oracle_convert_f32_to_f16.argtypes = [c_float_p, c_u16_p, sz, i]
         L.gm_oracle_convert_f32_to_f16.restype = None
         L.gm_oracle_convert_f16_to_f32.argtypes = [c_u16_p, c_float_p, sz, i]

@@ -1,5 +1,7 @@
 """Properties of the CPU oracle that the mathematics fixes (closed forms, invariants, library
 casts): a dropped term, a wrong sign or a misplaced epsilon fails one of them."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -268,3 +270,44 @@ def test_amp_scale_stays_finite_and_normal():
         scales.append(float(st.scale))
     assert scales == [2.0 ** -125, 2.0 ** -126, 2.0 ** -126, 2.0 ** -126, 2.0 ** -126]
     assert [s for _, s, _, _ in amp_reference_sequence([1] * 5, 2.0 ** -124, 2.0, 0.5, 1000)] == scales
+
+
+def test_fast_forms_of_the_fp16_conversions_equal_the_reference_forms_everywhere():
+    """The bulk loops convert through inlined fast paths; over all 2^32 binary32 patterns and all 2^16
+    binary16 patterns they return what gm_oracle_f32_to_f16 / gm_oracle_f16_to_f32 return (which are pinned
+    against numpy exhaustively / on boundary sets in tests/test_oracle_golden.py)."""
+    o = oracle()
+    threads = min(8, __import__("os").cpu_count() or 1)
+    assert o.lib.gm_oracle_f16_fast_mismatches(0, 1 << 32, 0, threads) == 0
+    assert o.lib.gm_oracle_f16_fast_mismatches(0, 1 << 16, 1, 1) == 0
+
+
+def test_vector_form_of_the_mixed_precision_step_equals_the_scalar_form():
+    """Hosts with AVX2 + F16C run the applied mixed-precision step eight lanes at a time.  Both forms over
+    the same inputs (every fp16 pattern as a gradient, inf and NaN included; weights and moments with random
+    bit patterns, subnormals, zeros, negative second moments) must agree in every bit of w, m, v and w16 (a NaN
+    result counts as equal to any NaN: payload propagation depends on operand order)."""
+    o = oracle()
+    rng = np.random.default_rng(99)
+    n = 1 << 18
+    g16 = np.tile(np.arange(1 << 16, dtype=np.uint16), n >> 16)
+    rng.shuffle(g16)
+    for case in range(4):
+        if case == 0:        # ordinary training data
+            w, m, v = rand(0.02, n), rand(1e-3, n), np.abs(rand(1e-6, n))
+        elif case == 1:      # anything at all
+            w, m, v = (rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32).view(np.float32) for _ in range(3))
+        elif case == 2:      # tiny values: subnormal moments and weights, underflowing fp16 copies
+            w, m, v = rand(1e-6, n), rand(1e-39, n), np.abs(rand(1e-42, n))
+        else:                # weights around the fp16 limits
+            w, m, v = rand(40000.0, n), rand(1e-3, n), np.abs(rand(1e-6, n))
+        for wd in (0.0, 1e-4):
+            bad = o.lib.gm_oracle_amp_vector_mismatches(
+                np.ascontiguousarray(w).ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                g16.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)),
+                np.ascontiguousarray(m).ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                np.ascontiguousarray(v).ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                n, 1e-3, 0.9, 0.999, 1e-8, wd, 0.1, 0.001, 1.0 / 65536.0)
+            if bad == 2 ** 64 - 1:
+                pytest.skip("this host has no AVX2 + F16C: the scalar form is the only one")
+            assert bad == 0, (case, wd, bad)
