@@ -11,6 +11,10 @@ the dominant kernel (algorithmic bytes per launch / launch duration measured wit
 events on the library's own stream, against MI355X's 8 TB/s HBM peak), the same figures for
 the mixed-precision (fp16 gradient) Adam step, and the CPU oracle timed on this host's cores
 on a bounded sample of the same workload.
+
+Without --workload, every benchmark configuration runs, each in a process of its own: the line
+is the headline configuration's, and "configs" holds the same record for configurations 1 to 4
+(--workload all adds the L-BFGS workloads and the buffer primitives; --workload NAME runs one).
 """
 import argparse
 import ctypes
@@ -35,8 +39,23 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
 MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10,
+                        # the three launches of one mixed-precision step: check 2.026e9 + update 2.8345e10
+                        ("c5", "adam_amp"): 3.0371e10,
                         # bytes per step, summed over the passes of a 10-pair step (profiles/lbfgs_c5_1b_hbm_traffic.md)
                         ("lbfgs-c5", 10): 352.68 * 1012301824}
+TRAFFIC_SOURCE = {("c5", "adam"): "profiles/adam_c5_1b_hbm_traffic.md",
+                  ("c5", "adam_amp"): "profiles/adam_c5_1b_hbm_traffic.md",
+                  ("lbfgs-c5", 10): "profiles/lbfgs_c5_1b_hbm_traffic.md"}
+
+
+def traffic_fields(key):
+    """roofline.traffic and where it comes from: HBM bytes per launch from separate rocprofv3 counter runs of this
+    file (FETCH_SIZE, then WRITE_SIZE), copied from the named summary; this run does not read counters."""
+    if key not in MEASURED_HBM_TRAFFIC:
+        return {"traffic": None, "traffic_source": "not measured for this workload"}
+    return {"traffic": MEASURED_HBM_TRAFFIC[key],
+            "traffic_source": f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, summary in "
+                              f"{TRAFFIC_SOURCE[key]}; a constant from that profile, not measured by this run"}
 
 from workloads import amp_125m_sizes, cnn_sizes, ragged_sizes, transformer_block_sizes  # noqa: E402
 
@@ -100,6 +119,41 @@ def per_launch_times(dev, launch, steps):
         launch()
         times.append(dev.lib.gm_timer_stop(dev.handle))
     return float(np.median(times)), float(min(times))
+
+
+def cpu_baseline_amp(sizes, hyper, grad_std, budget_params=96_000_000, target_seconds=3.0):
+    """The oracle's mixed-precision Adam step (clean steps: check, unscale, update, fp16 copy) on this host."""
+    from oracle_lib import oracle
+    o = oracle()
+    threads = min(16, os.cpu_count() or 1)
+    chosen, total = [], 0
+    for n in sizes:
+        if chosen and total + n > budget_params:
+            break
+        chosen.append(n)
+        total += n
+    rng = np.random.default_rng(2)
+    w = [rng.standard_normal(n, dtype=np.float32) * np.float32(0.02) for n in chosen]
+    m = [np.zeros(n, np.float32) for n in chosen]
+    v = [np.zeros(n, np.float32) for n in chosen]
+    w16 = [np.zeros(n, np.uint16) for n in chosen]
+    g16 = [(rng.standard_normal(n, dtype=np.float32) * np.float32(grad_std * 65536.0)).astype(np.float16).view(np.uint16)
+           for n in chosen]
+    st = o.amp_state(65536.0, 2.0, 0.5, 1 << 30)
+    step = lambda: o.adam_amp(w, g16, m, v, w16, state=st, nthreads=threads, **hyper)
+    step()
+    t0 = time.perf_counter()
+    step()
+    one = max(time.perf_counter() - t0, 1e-4)
+    steps = int(min(1_000_000, max(3, target_seconds / one)))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    dt = time.perf_counter() - t0
+    return {"value": total * steps / dt, "unit": "params/s", "cores": threads, "kind": "port",
+            "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} mixed-precision steps in "
+                      f"{dt:.1f} s, oracle/oracle.c (eight-lane AVX2 + F16C form where the host has them) with OpenMP "
+                      f"on {threads} threads of {os.cpu_count()} ({cpu_model()})"}
 
 
 def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_seconds=12.0):
@@ -216,7 +270,7 @@ def bench_lbfgs(args, pkg, dev):
         "vs_baseline": None, "dtype": "f32 (dot products accumulated in f64)", "data": "synthetic",
         "config": {"workload": desc, "tensors": n, "params": params, "rule": "lbfgs", "history_size": m},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_HBM_TRAFFIC.get((args.workload, m)),
+                     "frac": achieved / HBM_PEAK_GBS, **traffic_fields((args.workload, m)),
                      "kernel": "lbfgs_stream_kernel (all passes)",
                      "bytes_per_param": bpp, "kernel_ms": full_event,
                      "note": "time covers every pass of the step, the tree reductions between them and the "
@@ -295,7 +349,7 @@ def bench_primitives(args, pkg, dev):
     result["value"] = head["achieved"]
     result["ms_per_step"] = head["ms_per_call"]
     result["roofline"] = {"bound": "hbm", "achieved": head["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": head["frac"], "traffic": None, "kernel": "convert_f32_to_f16_kernel",
+                          "frac": head["frac"], **traffic_fields(None), "kernel": "convert_f32_to_f16_kernel",
                           "kernel_ms": head["kernel_ms"]}
     result["primitives"] = table
     result["host_copies"] = pcie
@@ -352,17 +406,25 @@ def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
                       f"runs this step as a single-threaded CPU loop); host: {cpu_model()}"}
 
 
-def run_all(args):
-    """Every configuration as a child process (this process never touches the GPU)."""
+BASELINE_CONFIGS = ["c5", "c1", "c2-sgd", "c2-adam", "c3-rmsprop", "c3-adagrad", "c3-adadelta", "c3-nadam", "c4"]
+
+
+def run_children(args, names):
+    """Each named workload as a child process, started before this process has made any GPU call (it never
+    makes one).  The line printed is the headline configuration's, with the others under "configs"."""
     import subprocess
     results = {}
-    for name in sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives"]:
+    for name in names:
         # Steps over the smaller lists take 5 to 500 us, and the first few hundred launches after the device
         # has been idle run slower: those workloads get at least 300 warm-up steps so that the timed ones
-        # show the kernels at their steady rate.
-        warmup = args.warmup if name in ("c5", "lbfgs-c5", "primitives") else max(args.warmup, 300)
-        cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", str(args.steps),
-               "--warmup", str(warmup)]
+        # show the kernels at their steady rate.  Their CPU samples are 3 s each, the headline's 12 s.
+        headline = name in ("c5", "lbfgs-c5", "primitives")
+        warmup = args.warmup if headline else max(args.warmup, 300)
+        # ... and at least 200 timed steps, so that the one wait at the end of the timed region (about 40 us)
+        # does not show in a per-step figure of a few microseconds; every record states its own counts
+        steps = args.steps if headline or name == "lbfgs-c3" else max(args.steps, 200)
+        cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", str(steps),
+               "--warmup", str(warmup), "--cpu-seconds", str(args.cpu_seconds if name == "c5" else min(args.cpu_seconds, 3.0))]
         if args.no_cpu_baseline:
             cmd.append("--no-cpu-baseline")
         print(f"running {name}", file=sys.stderr, flush=True)
@@ -378,9 +440,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives", "all"],
-                    help="'all': every configuration in turn, each in a process of its own; the line printed "
-                         "is the headline configuration's with the others under 'configs'")
+    ap.add_argument("--workload", default="", choices=[""] + sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives", "all"],
+                    help="one workload in this process.  Default: the five benchmark configurations in turn, each in a "
+                         "process of its own; the line printed is the headline configuration's (c5) with the others "
+                         "under 'configs'.  'all': the same plus the L-BFGS workloads and the buffer primitives")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU time of the oracle sample (cpu_baseline)")
+    ap.add_argument("--amp-check-order", default="", help="mixed-precision overflow check, for re-measurement: "
+                    "'NT,REV' with NT 1/0 = non-temporal loads on/off and REV 1/0 = walk the table backwards")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
     ap.add_argument("--history", type=int, default=0, help="L-BFGS workloads: history size (default 10)")
@@ -396,8 +462,10 @@ def main():
         sys.exit("bench.py measures one GPU: the optimizer step shards without communication, and this "
                  "build runs and reports a single MI355X (--gpus 1).")
 
+    if args.workload == "":
+        return run_children(args, BASELINE_CONFIGS)
     if args.workload == "all":
-        return run_all(args)
+        return run_children(args, BASELINE_CONFIGS + sorted(LBFGS_WORKLOADS) + ["primitives"])
 
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -407,6 +475,9 @@ def main():
         sys.exit("invalid --chunk / --vec combination (a chunk is a power-of-two multiple of 256 * vec elements)")
     if lib.gm_set_workgroup_lanes(args.lanes) != 0:
         sys.exit("invalid --lanes (128 or 256)")
+    if args.amp_check_order:
+        nt_flag, rev_flag = (int(x) for x in args.amp_check_order.split(","))
+        lib.gm_set_amp_check_order(nt_flag, rev_flag)
 
     if args.workload in LBFGS_WORKLOADS:
         return bench_lbfgs(args, pkg, dev)
@@ -473,8 +544,6 @@ def main():
     dev.free(src)
     dev.free(dst)
 
-    traffic = MEASURED_HBM_TRAFFIC.get((args.workload, rule))
-
     result = {
         "metric": "params updated/sec (Adam fp32 multi-tensor step) + achieved HBM GB/s (% of peak)"
                   if rule == "adam" else f"params updated/sec ({rule} multi-tensor step) + achieved HBM GB/s",
@@ -488,7 +557,7 @@ def main():
                    "launch": {"chunk": args.chunk or "auto", "vec": args.vec or "auto", "lanes": args.lanes or "auto",
                               "nontemporal": args.nontemporal != 0}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "frac": achieved / HBM_PEAK_GBS, **traffic_fields((args.workload, rule)),
                      "kernel": f"multi_tensor_update_kernel<{rule}>", "bytes_per_param": bpp,
                      "kernel_ms": event_ms, "kernel_ms_median": median_ms, "kernel_ms_min": min_ms,
                      "copy_kernel_gbs": copy_gbs,
@@ -525,7 +594,9 @@ def main():
             "dtype": "f32 master state, f16 gradients and weight copy", "skipped_steps": amp_t["skipped"],
             "roofline": {"bound": "hbm", "achieved": amp_achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": amp_achieved / HBM_PEAK_GBS, "bytes_per_param": 28,
-                         "bytes_per_param_moved": 30,
+                         "bytes_per_param_moved": 30, **traffic_fields((args.workload, "adam_amp")),
+                         "kernel": "amp_overflow_check_kernel + amp_adam_update_kernel + amp_finalize_kernel",
+                         "kernel_ms": amp_event,
                          "note": "step time covers the overflow-check launch, the update launch and the "
                                  "read-back of the skip flag; each step is synchronous"},
         }
@@ -547,11 +618,23 @@ def main():
             "note": "execute_adam_amp_step_async: no host wait per step; HIP-event time per step over the timed steps",
         }
         lib.gm_amp_state_destroy(amp)
+        if not args.no_cpu_baseline and args.workload in ("c4", "c5"):
+            result["amp"]["cpu_baseline"] = cpu_baseline_amp(sizes, hyper, grad_std, target_seconds=min(args.cpu_seconds, 3.0))
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(sizes, rule, hyper, grad_std)
+        result["cpu_baseline"] = cpu_baseline(sizes, rule, hyper, grad_std, target_seconds=args.cpu_seconds)
     else:
         result["cpu_baseline"] = None
+
+    if args.workload == "c4" and "amp" in result:
+        # configuration 4 IS the mixed-precision step: its figures lead, the fp32 step over the same list follows
+        amp_part = result.pop("amp")
+        fp32_part = {k: result[k] for k in ("value", "unit", "ms_per_step", "dtype", "roofline", "cpu_baseline")}
+        result.update({"metric": "params updated/sec (mixed-precision Adam step, fp16 gradients and weight copy) + "
+                                 "achieved HBM GB/s (% of peak)",
+                       "value": amp_part["value"], "ms_per_step": amp_part["ms_per_step"], "dtype": amp_part["dtype"],
+                       "roofline": amp_part["roofline"], "cpu_baseline": amp_part.get("cpu_baseline"),
+                       "skipped_steps": amp_part["skipped_steps"], "async": amp_part["async"], "fp32_adam": fp32_part})
 
     dev.close()
     print(json.dumps(result))

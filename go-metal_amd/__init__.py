@@ -78,6 +78,7 @@ ABI = {
     "gm_copy_probe": (i, [u, u, u, ctypes.c_size_t]),
     "gm_set_tuning": (i, [i, i, i]),
     "gm_set_workgroup_lanes": (i, [i]),
+    "gm_set_amp_check_order": (i, [i, i]),
 }
 
 # name -> (restype, argtypes): every symbol include/gometal_optimizer.h declares

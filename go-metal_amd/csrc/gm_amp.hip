@@ -15,6 +15,10 @@ namespace gm {
 
 constexpr float kMinLossScale = 1.17549435e-38f;   // FLT_MIN
 constexpr float kMaxLossScale = 3.40282347e+38f;   // FLT_MAX
+// Measurement switches of the overflow check (gm_set_amp_check_order): cache policy of its loads
+// and the direction it walks the table in.
+static std::atomic<int> g_check_nontemporal{1};
+static std::atomic<int> g_check_reverse{0};
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 
 // Loss-scale state machine, resident in HBM next to the tensors.
@@ -50,10 +54,12 @@ struct AmpBiasTable {
 // one atomic per workgroup that saw a hit.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
-amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state)
+amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state, int reverse)
 {
     __shared__ unsigned int wave_hit[kBlock / 64];
-    const Chunk ch = chunks[blockIdx.x];
+    // reverse: the table is walked from its end, so that the check finishes on the gradients the
+    // update pass reads first (what is left of them in the memory-side cache is then the nearest)
+    const Chunk ch = chunks[reverse ? gridDim.x - 1u - blockIdx.x : blockIdx.x];
     const unsigned short *g = reinterpret_cast<const unsigned short *>(ch.p[kSlotGrad]);
     unsigned int bad = 0;
     uint32_t done = 0;
@@ -244,6 +250,13 @@ static void amp_free(AmpState *s)
     delete s;
 }
 
+int gm_set_amp_check_order(int nontemporal, int reverse)
+{
+    g_check_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
+    g_check_reverse.store(reverse < 0 ? 0 : (reverse ? 1 : 0));
+    return 0;
+}
+
 uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth_factor,
                               float backoff_factor, int growth_interval)
 try {
@@ -418,8 +431,11 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
         int count;
         if (!launch_geometry(*l.plan, vec, block, seg, count)) return -6;
         // the check walks the whole table, one workgroup per chunk of either segment
-        if (nt) amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
-        else amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state);
+        const int reverse = g_check_reverse.load();
+        if (nt && g_check_nontemporal.load())
+            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse);
+        else
+            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse);
 #define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, amp->d_state, bias)
 #define GM_LAUNCH_AMP_B(B)                                                              \
         if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true, B); else GM_LAUNCH_AMP(4, false, B); }        \

@@ -364,6 +364,12 @@ int gm_set_tuning(int chunk_elements, int nontemporal, int vec);
  * five streams, else 256).  -1 on any other value (nothing changes). */
 int gm_set_workgroup_lanes(int lanes);
 
+/* The overflow check of the mixed-precision step, for re-measurement: whether its loads carry the
+ * non-temporal hint (default 1; -1 = default) and whether it walks the chunk table backwards, ending
+ * on the gradients the update pass reads first (default 0; -1 = default).  Results do not depend on
+ * either.  Always 0. */
+int gm_set_amp_check_order(int nontemporal, int reverse);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,7 +41,7 @@ def test_workload_lists_match_the_configurations():
 @pytest.mark.gpu
 def test_one_json_line_with_roofline_and_cpu_baseline():
     """A short run of a small workload prints exactly one line of JSON with the fields the driver reads."""
-    r = subprocess.run([sys.executable, BENCH, "--workload", "c2-adam", "--steps", "5", "--warmup", "2"],
+    r = subprocess.run([sys.executable, BENCH, "--workload", "c2-adam", "--steps", "5", "--warmup", "2", "--cpu-seconds", "2"],
                        capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if l.strip()]
@@ -55,5 +55,6 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     roof = j["roofline"]
     assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-12
+    assert "traffic" in roof and "not measured" in roof["traffic_source"]
     cpu = j["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
