@@ -395,3 +395,95 @@ def test_random_lists_histories_and_step_sizes(dev, seed):
             index, count = (index + 1) % m, min(count + 1, m)
     finally:
         run.free()
+
+
+def recursion_float64(g, s, y, rho, count, index, perturb=None):
+    """The two-loop recursion of the step (bridge_optimizer.m:1025-1213) in float64 with exact dot products,
+    on flat vectors.  perturb = (k, delta) adds delta to the k-th dot product taken.  Returns the direction p,
+    the alphas and, for every dot product, (value, sum of |a_i b_i|)."""
+    m = len(s)
+    q = -g.copy()
+    alpha = np.zeros(count)
+    dots = []
+
+    def dot(a, b):
+        k = len(dots)
+        value = float(np.dot(a, b))
+        dots.append((value, float(np.dot(np.abs(a), np.abs(b)))))
+        return value + (perturb[1] if perturb and perturb[0] == k else 0.0)
+
+    for j in range(count - 1, -1, -1):
+        idx = (index - count + j + m) % m
+        if abs(rho[idx]) < 1e-10:
+            continue
+        alpha[j] = rho[idx] * dot(s[idx], q)
+        q = q - alpha[j] * y[idx]
+    for j in range(count):
+        idx = (index - count + j + m) % m
+        if abs(rho[idx]) < 1e-10:
+            continue
+        beta = rho[idx] * dot(y[idx], q)
+        q = q + (alpha[j] - beta) * s[idx]
+    return -q, alpha, dots
+
+
+def test_step_against_the_reference_summation_order_within_the_propagated_bound(dev):
+    """The reference sums each dot product as a running fp32 sum in element order (bridge_optimizer.m:1100-1104);
+    the library sums exact fp64 products in a fixed tree.  The two orders cannot agree bit for bit, so the GPU step
+    is compared with the oracle run in the REFERENCE order under a stated bound: a running fp32 sum of n terms is
+    within gamma_n * sum|a_i b_i| of the exact dot product (gamma_n = n u / (1 - n u), u = 2^-24), the tree within
+    half an fp32 ulp.  That per-dot error is pushed through the recursion numerically (each dot product of a float64
+    model of the recursion shifted by its own bound, one at a time, both signs) and the shifts of every alpha and
+    every element of the direction are added up: twice that sum, plus a few ulps for the elementwise fp32 roundings,
+    bounds the distance between the two runs.  The bound is tight enough to notice a missing term: it stays below
+    2 % of the direction's largest element."""
+    sizes, m, count, index = [70_000, 5, 4097, 1023, 30_000], 4, 3, 3
+    rng = np.random.default_rng(77)
+    r = lambda k, scale: (rng.standard_normal(k) * scale).astype(F)
+    st = {"w": [r(k, 0.5) for k in sizes], "old_g": [r(k, 1e-2) for k in sizes], "dir": [np.zeros(k, F) for k in sizes],
+          "s": [[r(k, 1e-2) for k in sizes] for _ in range(m)], "y": [[r(k, 1e-2) for k in sizes] for _ in range(m)],
+          "rho": np.zeros(m, F), "alpha": np.zeros(m, F)}
+    flat = lambda ts: np.concatenate([t.astype(np.float64) for t in ts])
+    # rho_j = 1 / (s_j . y_j'), with y_j' = y_j + 3 s_j so that the curvature is positive and alpha is O(1)
+    for h in range(m):
+        st["y"][h] = [(yt + F(3.0) * st_).astype(F) for yt, st_ in zip(st["y"][h], st["s"][h])]
+        st["rho"][h] = F(1.0 / np.dot(flat(st["s"][h]), flat(st["y"][h])))
+    g = [r(k, 1e-2) for k in sizes]
+    ref = clone(st)
+    run = LbfgsGpu(dev, st)
+    try:
+        run.step(g, count, index, 0.5)
+        got = run.download()
+    finally:
+        run.free()
+    assert oracle().lbfgs_step(ref, g, m, count, index, 0.5, 0)[0] == 0          # 0: the reference's own order
+
+    gf, sf, yf = flat(g), [flat(h) for h in st["s"]], [flat(h) for h in st["y"]]
+    rho = st["rho"].astype(np.float64)
+    p0, alpha0, dots = recursion_float64(gf, sf, yf, rho, count, index)
+    assert len(dots) == 2 * count
+    n, u = gf.size + len(sizes), 2.0 ** -24
+    gamma = n * u / (1 - n * u)
+    bound_p, bound_alpha = np.zeros_like(p0), np.zeros(count)
+    for k, (value, magnitude) in enumerate(dots):
+        e = gamma * magnitude + abs(value) * u             # running-sum bound, plus the final rounding of either order
+        shift_p, shift_a = np.zeros_like(p0), np.zeros(count)
+        for sign in (1.0, -1.0):
+            p1, alpha1, _ = recursion_float64(gf, sf, yf, rho, count, index, perturb=(k, sign * e))
+            shift_p, shift_a = np.maximum(shift_p, np.abs(p1 - p0)), np.maximum(shift_a, np.abs(alpha1 - alpha0))
+        bound_p += shift_p
+        bound_alpha += shift_a
+    ulps = 32 * u
+    slack_p = ulps * (np.abs(p0) + np.abs(gf) + sum(abs(a) * np.abs(yv) for a, yv in zip(alpha0, yf[:count])) +
+                      sum((abs(a) + 1.0) * np.abs(sv) for a, sv in zip(alpha0, sf)))
+    assert bound_p.max() < 0.02 * np.abs(p0).max(), "the bound must stay small against the direction itself"
+
+    p_gpu, p_ref = flat(got["dir"]), flat(ref["dir"])
+    assert not np.array_equal(p_gpu, p_ref), "the two summation orders are expected to differ in the last bits"
+    assert np.all(np.abs(p_gpu - p_ref) <= 2 * bound_p + slack_p)
+    assert np.all(np.abs(p_gpu - p0) <= bound_p + slack_p) and np.all(np.abs(p_ref - p0) <= bound_p + slack_p)
+    a_gpu, a_ref = got["alpha"][:count].astype(np.float64), ref["alpha"][:count].astype(np.float64)
+    assert np.all(np.abs(a_gpu - a_ref) <= 2 * bound_alpha + ulps * np.abs(alpha0))
+    # the weights moved by step * p in both runs
+    w_gpu, w_ref = flat(got["w"]), flat(ref["w"])
+    assert np.all(np.abs(w_gpu - w_ref) <= 0.5 * (2 * bound_p + slack_p) + 4 * u * np.abs(w_ref))
