@@ -8,7 +8,9 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
-ORACLE_SO = os.path.join(ORACLE_DIR, "liboracle.so")
+# GM_ORACLE_SO points the tests at another build of the checker: how a deliberately perturbed oracle.c is
+# shown to fail the pins in tests/test_oracle_properties.py
+ORACLE_SO = os.environ.get("GM_ORACLE_SO") or os.path.join(ORACLE_DIR, "liboracle.so")
 
 c_float_p = ctypes.POINTER(ctypes.c_float)
 c_u16_p = ctypes.POINTER(ctypes.c_uint16)

@@ -311,3 +311,160 @@ def test_vector_form_of_the_mixed_precision_step_equals_the_scalar_form():
             if bad == 2 ** 64 - 1:
                 pytest.skip("this host has no AVX2 + F16C: the scalar form is the only one")
             assert bad == 0, (case, wd, bad)
+
+
+# ---- pins that separate neighbouring formulas (each docstring names the perturbation of oracle.c it was
+# ---- checked against: the test fails with that one line changed and passes with the line as it is)
+F = np.float32
+
+
+def nadam_mu_float64(beta1, t):
+    """bridge_optimizer.m:2066 in float64: beta1 * (1 - 0.5 * 0.96^((t + 1) * 0.004))."""
+    return float(F(beta1)) * (1.0 - 0.5 * 0.96 ** ((t + 1) * 0.004))
+
+
+def test_nadam_momentum_schedule_is_taken_at_t_plus_one():
+    """mu(t + 1), not mu(t): the two differ by 8e-5 relative, a thousand times the tolerance used here.
+    Perturbation tried: `(float)(step + 1)` -> `(float)step` in gm_oracle_nadam_mu_next: fails at every t."""
+    o = oracle()
+    for t in (1, 2, 10, 250, 2500, 5000):
+        got = float(o.nadam_mu_next(0.9, t))
+        assert abs(got - nadam_mu_float64(0.9, t)) <= 2e-7 * abs(got), t
+        assert abs(got - float(F(0.9)) * (1.0 - 0.5 * 0.96 ** (t * 0.004))) > 1e-5 * abs(got), t
+    # and the schedule really moves between steps 1 and 250 (a constant mu would pass the check above at one t)
+    assert float(o.nadam_mu_next(0.9, 250)) - float(o.nadam_mu_next(0.9, 1)) > 0.9 * 0.5 * 0.035
+
+
+def nadam_first_step_float32(w, g, lr, b1, b2, eps, wd, mu):
+    """t = 1, m = v = 0: every operation of bridge_optimizer.m:2114-2198 as one numpy float32 operation."""
+    lr, b1, b2, eps, wd, mu = (F(x) for x in (lr, b1, b2, eps, wd, mu))
+    one = F(1.0)
+    bc1, bc2 = one - b1, one - b2                       # 1 - beta^1
+    m = g * (one - b1)                                  # :2117-2120 with m = 0 (0 * beta1 + x = x exactly)
+    v = (g * g) * (one - b2)                            # :2125-2134
+    v_hat, m_hat, g_hat = v / bc2, m / bc1, g / bc1     # :2139-2148
+    m_bar = m_hat * mu + g_hat * (one - mu)             # :2158-2164
+    den = np.sqrt(v_hat) + eps                          # :2170-2171  epsilon OUTSIDE the root
+    upd = m_bar / den                                   # :2176
+    if wd > 0:
+        upd = upd + w * wd                              # :2181-2190  decay after the adaptive term, on the old weight
+    return w - upd * lr, m, v                           # :2193-2198
+
+
+@pytest.mark.parametrize("wd", [0.0, 0.01])
+def test_nadam_first_step_closed_form_bit_exact(wd):
+    """First step against a chain of numpy float32 operations, with and without weight decay, on gradients
+    spread over twelve decades (so that v_hat ranges from far below eps^2 to far above).
+    Perturbations tried, each failing this test: eps moved inside the root (`sqrtf(v_hat + eps)`), `g_term`
+    dropped from m_bar, decay added to the gradient instead of the update."""
+    o = oracle()
+    w = rand(0.5)
+    g = (rand(1.0) * F(10.0) ** RNG.integers(-10, 2, N).astype(F)).astype(F)
+    w0 = w.copy()
+    m, v = np.zeros(N, F), np.zeros(N, F)
+    o.nadam(w, g, m, v, 0.002, 0.9, 0.999, 1e-8, wd, 1)
+    want_w, want_m, want_v = nadam_first_step_float32(w0, g, 0.002, 0.9, 0.999, 1e-8, wd, o.nadam_mu_next(0.9, 1))
+    assert np.array_equal(m.view(np.uint32), want_m.view(np.uint32))
+    assert np.array_equal(v.view(np.uint32), want_v.view(np.uint32))
+    assert np.array_equal(w.view(np.uint32), want_w.view(np.uint32))
+
+
+def test_epsilon_placement_where_it_decides_the_result():
+    """Gradients of 1e-8, where sqrt(v_hat) equals eps: with eps outside the root the denominator is 2e-8,
+    with eps inside it would be 1e-4, a factor of 5000 in the step.  Adam and NAdam put eps outside
+    (bridge_optimizer.m:519-521, :2170-2171); RMSProp puts it inside (:827-830).
+    Perturbations tried: Adam `sqrtf(v_hat) + eps` -> `sqrtf(v_hat + eps)`, the same for NAdam, and RMSProp
+    `sqrtf(s_eps)` -> `sqrtf(si) + eps`: each fails its assertion below."""
+    o = oracle()
+    g = np.full(N, 1e-8, F)
+    g[::2] *= F(-1)
+    # Adam, t = 1: m_hat = g, v_hat = g^2  ->  step = lr * g / (|g| + eps) = lr / 2
+    w, m, v = np.zeros(N, F), np.zeros(N, F), np.zeros(N, F)
+    o.adam(w, g, m, v, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1)
+    np.testing.assert_allclose(np.abs(w), 0.5e-3, rtol=1e-5)
+    # NAdam, t = 1: m_bar = (mu + 10 (1 - mu)) g
+    w, m, v = np.zeros(N, F), np.zeros(N, F), np.zeros(N, F)
+    o.nadam(w, g, m, v, 0.002, 0.9, 0.999, 1e-8, 0.0, 1)
+    mu = nadam_mu_float64(0.9, 1)
+    np.testing.assert_allclose(np.abs(w), 0.002 * (mu + 10 * (1 - mu)) / 2, rtol=1e-4)
+    # RMSProp: s = 0.01 g^2 = 1e-18, root = sqrt(1e-18 + 1e-8) ~ 1e-4  ->  step = lr * g / 1e-4 = 1e-6
+    w, s = np.zeros(N, F), np.zeros(N, F)
+    o.rmsprop(w, g, s, None, None, 0.01, 0.99, 1e-8, 0.0, 0.0, False)
+    np.testing.assert_allclose(np.abs(w), 0.01 * 1e-8 / 1e-4, rtol=1e-4)
+
+
+def test_adadelta_second_step_uses_the_previous_update_average():
+    """Two steps as numpy float32 chains: the step-2 numerator is sqrt(E[dx^2] + eps) with the average as it
+    stood BEFORE step 2 (bridge_optimizer.m:1807-1810 reads the buffer, :1832-1841 writes it afterwards).
+    Only visible from the second step on (the first starts from zero either way).
+    Perturbations tried: the update average advanced before rms_u is formed (which no first-step test can
+    see), and rho used in place of (1 - rho) in the update average: both fail here."""
+    o = oracle()
+    rho, eps, one = F(0.9), F(1e-6), F(1.0)
+    w, s, a = rand(0.1), np.zeros(N, F), np.zeros(N, F)
+    ws, ss, as_ = w.copy(), s.copy(), a.copy()
+    for step in range(2):
+        g = rand(1e-2)
+        o.adadelta(w, g, s, a, 0.9, 1e-6, 0.0)
+        s_new = ss * rho + (g * g) * (one - rho)
+        d = (np.sqrt(as_ + eps) / np.sqrt(s_new + eps)) * g          # as_ is the OLD average
+        neg_d = -d
+        ws = ws + neg_d
+        as_ = as_ * rho + (neg_d * neg_d) * (one - rho)
+        ss = s_new
+        for got, want, name in ((w, ws, "w"), (s, ss, "s"), (a, as_, "a")):
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (step, name)
+    assert np.all(a > 0)
+
+
+def test_decay_order_for_every_rule_on_a_zero_gradient():
+    """With g = 0 a rule that adds the decay to the UPDATE (Adam, NAdam, RMSProp: bridge_optimizer.m:531-540,
+    :2181-2190, :857-866) moves w by exactly lr * (w * wd) and leaves every state at zero; a rule that adds it
+    to the GRADIENT (SGD, AdaGrad, AdaDelta: :219-228, :1480-1488, :1773-1781) feeds it through its state.
+    Perturbations tried: RMSProp and NAdam decay moved in front of the state update (`gi = gi + decay`): their
+    state assertions fail; AdaGrad decay moved behind the adaptive term: its state assertion fails."""
+    o = oracle()
+    lr, wd = F(0.01), F(0.1)
+    zero = np.zeros(N, F)
+    w0 = rand(0.5)
+    moved = w0 - (w0 * wd) * lr
+    # decay on the update
+    w, m, v = w0.copy(), zero.copy(), zero.copy()
+    o.adam(w, zero, m, v, 0.01, 0.9, 0.999, 1e-8, 0.1, 1)
+    assert np.array_equal(w, moved) and not m.any() and not v.any()
+    w, m, v = w0.copy(), zero.copy(), zero.copy()
+    o.nadam(w, zero, m, v, 0.01, 0.9, 0.999, 1e-8, 0.1, 1)
+    assert np.array_equal(w, moved) and not m.any() and not v.any()
+    w, s = w0.copy(), zero.copy()
+    o.rmsprop(w, zero, s, None, None, 0.01, 0.99, 1e-8, 0.1, 0.0, False)
+    assert np.array_equal(w, moved) and not s.any()
+    # decay into the gradient
+    gd = w0 * wd
+    w, s = w0.copy(), zero.copy()
+    o.adagrad(w, zero, s, 0.01, 1e-10, 0.1)
+    assert np.array_equal(s, gd * gd)
+    assert np.array_equal(w, w0 - (lr / (np.sqrt(gd * gd) + F(1e-10))) * gd)
+    w, s, a = w0.copy(), zero.copy(), zero.copy()
+    o.adadelta(w, zero, s, a, 0.9, 1e-6, 0.1)
+    assert np.array_equal(s, (gd * gd) * (F(1.0) - F(0.9)))
+    w, m = w0.copy(), zero.copy()
+    o.sgd(w, zero, m, 0.01, 0.9, 0.1, False)
+    assert np.array_equal(m, gd) and np.array_equal(w, w0 - lr * gd)
+
+
+def test_rmsprop_second_step_with_decay_bit_exact():
+    """Two plain RMSProp steps with weight decay as numpy float32 chains (bridge_optimizer.m:782-874): the
+    running average multiplies the OLD state by alpha and the new square by (1 - alpha); the decay joins the
+    update after the division.  Perturbation tried: alpha and (1 - alpha) swapped: fails at step 1."""
+    o = oracle()
+    alpha, eps, lr, wd, one = F(0.99), F(1e-8), F(0.01), F(1e-2), F(1.0)
+    w, s = rand(0.5), np.zeros(N, F)
+    ws, ss = w.copy(), s.copy()
+    for step in range(2):
+        g = rand(1e-2)
+        o.rmsprop(w, g, s, None, None, 0.01, 0.99, 1e-8, 1e-2, 0.0, False)
+        ss = ss * alpha + (g * g) * (one - alpha)
+        upd = g / np.sqrt(ss + eps) + ws * wd
+        ws = ws - upd * lr
+        assert np.array_equal(s.view(np.uint32), ss.view(np.uint32)), step
+        assert np.array_equal(w.view(np.uint32), ws.view(np.uint32)), step
