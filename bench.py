@@ -618,6 +618,52 @@ def main():
             "note": "execute_adam_amp_step_async: no host wait per step; HIP-event time per step over the timed steps",
         }
         lib.gm_amp_state_destroy(amp)
+
+        # ---- the same step in one pass over ping-pong state (two sets of weights and moments) ----
+        shadow = [[dev.alloc(4 * s) for s in sizes] for _ in range(3)]
+        c_shadow = [pkg.handle_array(hs) for hs in shadow]
+        amp2 = lib.gm_amp_state_create(D, 65536.0, 2.0, 0.5, 2000)
+        lib.gm_amp_state_set_step_count(amp2, amp_t["t"])
+        cur = ctypes.c_int()
+        fused_t = {"t": amp_t["t"], "skipped": 0}
+
+        def launch_fused():
+            rc = lib.execute_adam_amp_step_fused(D, cw, cs[0], cs[1], c_shadow[0], c_shadow[1], c_shadow[2], cg16, cw16, n,
+                                                 bs, hyper["lr"], hyper["beta1"], hyper["beta2"], hyper["eps"],
+                                                 hyper["weight_decay"], fused_t["t"] + 1, amp2, ctypes.byref(skipped),
+                                                 ctypes.byref(scale), ctypes.byref(tracker), ctypes.byref(cur))
+            if rc != 0:
+                raise RuntimeError(f"one-pass mixed-precision step failed rc={rc}: {lib.gm_last_error().decode()}")
+            fused_t["skipped" if skipped.value else "t"] += 1
+
+        def launch_fused_async():
+            rc = lib.execute_adam_amp_step_fused_async(D, cw, cs[0], cs[1], c_shadow[0], c_shadow[1], c_shadow[2], cg16,
+                                                       cw16, n, bs, hyper["lr"], hyper["beta1"], hyper["beta2"],
+                                                       hyper["eps"], hyper["weight_decay"], amp2)
+            if rc != 0:
+                raise RuntimeError(f"one-pass asynchronous step failed rc={rc}: {lib.gm_last_error().decode()}")
+
+        fused_wall, fused_event = time_steps(dev, launch_fused, args.steps, args.warmup)
+        fa_wall, fa_event = time_steps(dev, launch_fused_async, args.steps, args.warmup)
+        fused_achieved = params * 28 / (fused_wall * 1e-3) / 1e9
+        fa_achieved = params * 28 / (fa_event * 1e-3) / 1e9
+        result["amp"]["one_pass"] = {
+            "entry_point": "execute_adam_amp_step_fused",
+            "value": params / (fused_wall * 1e-3), "unit": "params/s", "ms_per_step": fused_wall,
+            "skipped_steps": fused_t["skipped"],
+            "roofline": {"bound": "hbm", "achieved": fused_achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": fused_achieved / HBM_PEAK_GBS, "bytes_per_param": 28, "bytes_per_param_moved": 28,
+                         **traffic_fields((args.workload, "adam_amp_one_pass")),
+                         "kernel": "amp_adam_fused_kernel + amp_finalize_kernel + amp_repair_weight16_kernel",
+                         "kernel_ms": fused_event,
+                         "note": "weights and moments kept twice (ping-pong): the step reads the current set and "
+                                 "writes the other, so a dropped step needs no second read of the gradients; each "
+                                 "step is synchronous"},
+            "async": {"value": params / (fa_wall * 1e-3), "unit": "params/s", "ms_per_step": fa_wall,
+                      "kernel_ms": fa_event, "achieved": fa_achieved, "frac": fa_achieved / HBM_PEAK_GBS,
+                      "max_steps_in_flight": lib.gm_amp_state_max_in_flight(amp2)},
+        }
+        lib.gm_amp_state_destroy(amp2)
         if not args.no_cpu_baseline and args.workload in ("c4", "c5"):
             result["amp"]["cpu_baseline"] = cpu_baseline_amp(sizes, hyper, grad_std, target_seconds=min(args.cpu_seconds, 3.0))
 
@@ -634,7 +680,8 @@ def main():
                                  "achieved HBM GB/s (% of peak)",
                        "value": amp_part["value"], "ms_per_step": amp_part["ms_per_step"], "dtype": amp_part["dtype"],
                        "roofline": amp_part["roofline"], "cpu_baseline": amp_part.get("cpu_baseline"),
-                       "skipped_steps": amp_part["skipped_steps"], "async": amp_part["async"], "fp32_adam": fp32_part})
+                       "skipped_steps": amp_part["skipped_steps"], "async": amp_part["async"],
+                       "one_pass": amp_part["one_pass"], "fp32_adam": fp32_part})
 
     dev.close()
     print(json.dumps(result))

@@ -2,8 +2,19 @@
 // copy, loss-scale state machine; synchronous and run-ahead entry points.
 //
 // An inf in the last tensor must suppress the write to the first, and the Adam update is not
-// exactly invertible, so one pass cannot both check and write: the step is two streaming launches
-// plus a one-lane epilogue, all on one stream.
+// exactly invertible.  Two forms follow from that:
+//
+// in place (execute_adam_amp_step[_async]): weights and moments are updated where they lie, so
+//   nothing may be written before every gradient has been checked: a check launch reads the fp16
+//   gradients, an update launch reads them again (30 bytes move per parameter for 28 algorithmic
+//   ones), a one-lane epilogue advances the loss-scale state.
+// ping-pong (execute_adam_amp_step_fused[_async]): weights and moments exist twice (sets A and B),
+//   one of them current.  ONE launch reads the current set and the gradients, checks the
+//   gradients as it goes, and writes the other set; the epilogue makes that set current only if
+//   no gradient overflowed.  A dropped step leaves the current set untouched because it was
+//   never written: every stream moves once, 28 bytes per parameter.  The fp16 weight copy has a
+//   single consumer-visible buffer and is written speculatively; after a dropped step a repair
+//   pass (which returns at once after an applied one) rewrites it from the current weights.
 #include "gm_launch.hpp"
 #include "gm_update_kernels.hpp"
 
@@ -24,19 +35,21 @@ constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in
 // Loss-scale state machine, resident in HBM next to the tensors.
 struct alignas(16) AmpDeviceState {
     // head: the 16 bytes every workgroup of the update kernel reads with one scalar load
-    float scale;
+    int current_set;        // ping-pong step: 0 = set A holds the current weights and moments, 1 = set B
     float inv_scale;        // 1.0f / scale, kept by whoever changes scale (IEEE division on host and device alike)
-    int found_inf;          // set by the check kernel, consumed and cleared by the epilogue
+    int found_inf;          // set by the check (or the fused update), consumed and cleared by the epilogue
     int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
     // tail
+    float scale;
     int growth_tracker;
     int last_skipped;
     float growth_factor;
     float backoff_factor;
     int growth_interval;
     int skipped_steps;      // steps dropped so far
-    int pad[2];
+    int pad;
 };
+static_assert(sizeof(AmpDeviceState) == 48, "AmpDeviceState layout");
 
 // Bias corrections for the asynchronous step.  The host does not know how many of the steps
 // still in flight were applied, so it sends the corrections (glibc powf, like every other
@@ -105,7 +118,7 @@ __global__ void __launch_bounds__(BLOCK)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
                        const AmpDeviceState *__restrict__ state, AmpBiasTable bias)
 {
-    // The state's head (scale, its reciprocal, flag, applied steps) comes with one 16-byte scalar load
+    // The state's head (current set, reciprocal of the scale, flag, applied steps) comes with one 16-byte scalar load
     // and the chunk descriptor with another, both issued before anything is decided; the bias
     // table sits in the kernel arguments and its entry is picked by scalar selects.  No load
     // waits for another except on the kernel-argument pointers themselves.
@@ -133,11 +146,117 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     update_slice<AdamRule, VEC, NT, true, BLOCK>(ch, slice_shift, prm, inv_scale);
 }
 
+// The ping-pong step: one pass.  Reads weights and moments of the current set and the fp16
+// gradients, writes the other set and the fp16 weight copy, and raises the flag when a gradient
+// of its own is +-inf or NaN.  It never looks at the flag: what it writes becomes current only if
+// the epilogue finds the flag clear.
+template <int N, bool NT>
+__device__ inline bool amp_fused_group(const Chunk &in, const Chunk &out, uint32_t first, const StepParams &prm,
+                                       float inv_scale)
+{
+    typedef typename VecOf<float, N>::type FV;
+    typedef typename VecOf<unsigned short, N>::type UV;
+    typedef typename VecOf<_Float16, N>::type HV;
+    const FV W = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotWeight]) + first));
+    const UV H = stream_load<NT>(reinterpret_cast<const UV *>(reinterpret_cast<const unsigned short *>(in.p[kSlotGrad]) + first));
+    const FV M = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotState0]) + first));
+    const FV V = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotState1]) + first));
+    FV Wn, Mn, Vn;
+    HV Hn;
+    bool bad = false;
+#pragma unroll
+    for (int c = 0; c < N; c++) {
+        const unsigned short bits = lane_of<N>(H, c);
+        bad |= (bits & 0x7C00u) == 0x7C00u;
+        float wv = lane_of<N>(W, c);
+        float sv[2] = {lane_of<N>(M, c), lane_of<N>(V, c)};
+        const float gv = (float)__builtin_bit_cast(_Float16, bits) * inv_scale;
+        AdamRule::apply(wv, gv, sv, prm);
+        set_lane<N>(Wn, c, wv);
+        set_lane<N>(Mn, c, sv[0]);
+        set_lane<N>(Vn, c, sv[1]);
+        set_lane<N>(Hn, c, (_Float16)wv);
+    }
+    stream_store<NT>(Wn, reinterpret_cast<FV *>(reinterpret_cast<float *>(out.p[kSlotWeight]) + first));
+    stream_store<NT>(Mn, reinterpret_cast<FV *>(reinterpret_cast<float *>(out.p[kSlotState0]) + first));
+    stream_store<NT>(Vn, reinterpret_cast<FV *>(reinterpret_cast<float *>(out.p[kSlotState1]) + first));
+    if (out.p[kSlotWeight16])
+        stream_store<NT>(Hn, reinterpret_cast<HV *>(reinterpret_cast<_Float16 *>(out.p[kSlotWeight16]) + first));
+    return bad;
+}
+
+template <int VEC, bool NT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+amp_adam_fused_kernel(const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t slice_shift,
+                      StepParams prm, AmpDeviceState *__restrict__ state, AmpBiasTable bias)
+{
+    // three scalar loads issued together: the state's head and the chunk's descriptor in either set
+    const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
+    const uint32_t c = blockIdx.x >> slice_shift;
+    const Chunk a = set_a[c];
+    const Chunk b = set_b[c];
+    const uint32_t slice = blockIdx.x & ((1u << slice_shift) - 1u);
+    if ((slice * BLOCK * VEC >= a.count) | (a.p[kSlotWeight] == nullptr) | (b.p[kSlotWeight] == nullptr)) return;
+    const bool b_is_current = head.x != 0u;
+    const Chunk &in = b_is_current ? b : a;
+    const Chunk &out = b_is_current ? a : b;
+    const float inv_scale = __uint_as_float(head.y);
+    const int applied = (int)head.w;
+    int pick = bias.count > 1 ? applied - bias.base : 0;
+    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
+    float bc1 = bias.bc1[0], bc2 = bias.bc2[0];
+#pragma unroll
+    for (int j = 1; j < kAmpMaxInFlight; j++) {
+        if (pick == j) {
+            bc1 = bias.bc1[j];
+            bc2 = bias.bc2[j];
+        }
+    }
+    prm.bc1 = bc1;
+    prm.bc2 = bc2;
+    // vec-wide lanes need both sets aligned for them
+    const LaneShare s = lane_share(a.count, a.flags & b.flags, slice, threadIdx.x, VEC, BLOCK);
+    bool bad = false;
+    if (s.count != 0) {
+        if (VEC > 1 && s.grouped) {
+            bad = amp_fused_group<VEC, NT>(in, out, s.first, prm, inv_scale);
+        } else {
+            for (uint32_t e = 0; e < s.count; e++) bad |= amp_fused_group<1, NT>(in, out, s.first + e, prm, inv_scale);
+        }
+    }
+    // One atomic per wavefront that saw a hit, and none once the flag is up (a tensor of nothing but
+    // inf would otherwise send millions of atomics to one address).
+    const unsigned long long hit = __ballot(bad);
+    if (hit != 0ull && (threadIdx.x & 63u) == (unsigned int)(__ffsll((long long)hit) - 1) &&
+        __hip_atomic_load(&state->found_inf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+        atomicOr(&state->found_inf, 1);
+}
+
+// After a dropped ping-pong step the fp16 weight copy holds what the discarded update wrote:
+// it is rewritten from the current weights (the copy of an applied step is half(w) by
+// construction, so this restores it bit for bit).  Launched after the epilogue of every
+// ping-pong step on a small fixed grid; after an applied step every workgroup returns on its
+// first load.
+__global__ void __launch_bounds__(kBlock)
+amp_repair_weight16_kernel(const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t num_chunks,
+                           const AmpDeviceState *__restrict__ state)
+{
+    if (state->last_skipped == 0) return;
+    const Chunk *current = state->current_set != 0 ? set_b : set_a;
+    for (uint32_t c = blockIdx.x; c < num_chunks; c += gridDim.x) {
+        const Chunk ch = current[c];
+        if (ch.p[kSlotWeight16] == nullptr) continue;
+        const float *w = reinterpret_cast<const float *>(ch.p[kSlotWeight]);
+        _Float16 *h = reinterpret_cast<_Float16 *>(ch.p[kSlotWeight16]);
+        for (uint32_t e = threadIdx.x; e < ch.count; e += kBlock) h[e] = (_Float16)w[e];
+    }
+}
+
 // Epilogue (one lane, same stream, after phase B has drained): advances the
 // loss-scale state machine and re-arms the flag.  A separate launch rather
 // than a last-workgroup ticket: a single counter bumped by every workgroup of
 // a 250k-workgroup grid serialises in the memory-side atomic unit.
-__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror)
+__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror, int ping_pong)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     AmpDeviceState st = *state;
@@ -153,6 +272,7 @@ __global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_
         st.skipped_steps += 1;
     } else {
         st.applied_steps += 1;
+        if (ping_pong) st.current_set ^= 1;      // the set just written is the current one from here on
         st.growth_tracker += 1;
         if (st.growth_tracker == st.growth_interval) {
             const float next = st.scale * st.growth_factor;
@@ -365,13 +485,46 @@ try {
     return -6;
 }
 
-// Plan, parameters and the three launches shared by the synchronous and the asynchronous step.
-static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffers,
-                       uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
-                       uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
-                       int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
-                       float weight_decay, int step_count, bool async, Launch &l,
-                       std::unique_lock<std::mutex> &lock)
+static StepParams amp_step_params(float learning_rate, float beta1, float beta2, float epsilon, float weight_decay)
+{
+    StepParams p = zero_params();
+    p.lr = learning_rate;
+    p.beta1 = beta1;
+    p.beta2 = beta2;
+    p.one_minus_beta1 = 1.0f - beta1;
+    p.one_minus_beta2 = 1.0f - beta2;
+    p.eps = epsilon;
+    p.weight_decay = weight_decay;
+    return p;
+}
+
+// Bias corrections and the pinned slot this step's post-state goes to.  The context lock is held:
+// the issue counters of the loss-scale state are only read and advanced under it.  An asynchronous
+// step's post-state goes into the ring slot of its issue number, a synchronous step's into slot 0.
+static bool amp_bias_and_mirror(AmpState *amp, bool async, float beta1, float beta2, int step_count,
+                                AmpBiasTable &bias, AmpDeviceState *&host_mirror)
+{
+    host_mirror = amp->h_pinned;
+    bias = AmpBiasTable{};
+    if (async) {
+        if (!amp_poll(amp, true)) return false;
+        host_mirror = &amp->h_pinned[1 + (amp->issued + 1) % kAmpMaxInFlight];
+        const int in_flight = (int)(amp->issued - amp->confirmed_issue);
+        if (in_flight > amp->max_in_flight) amp->max_in_flight = in_flight;
+        bias.base = amp->confirmed_applied;
+        bias.count = in_flight + 1;
+        for (int j = 0; j <= in_flight; j++)
+            gm_bias_corrections(beta1, beta2, amp->confirmed_applied + 1 + j, &bias.bc1[j], &bias.bc2[j]);
+    } else {
+        bias.count = 1;
+        gm_bias_corrections(beta1, beta2, step_count, &bias.bc1[0], &bias.bc2[0]);
+    }
+    return true;
+}
+
+static PlanRequest amp_request(uintptr_t *weight_buffers, uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                               uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
+                               int *buffer_sizes)
 {
     PlanRequest req{};
     req.kind = kRuleAdamAMP;
@@ -385,39 +538,28 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     req.required_mask = (1u << kSlotWeight) | (1u << kSlotGrad) | (1u << kSlotState0) | (1u << kSlotState1);
     req.missing_code = -4;
     req.half_mask = (1u << kSlotGrad) | (1u << kSlotWeight16);
+    return req;
+}
+
+// Plan, parameters and the three launches shared by the synchronous and the asynchronous in-place step.
+static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffers,
+                       uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
+                       uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
+                       int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
+                       float weight_decay, int step_count, bool async, Launch &l,
+                       std::unique_lock<std::mutex> &lock)
+{
+    const PlanRequest req = amp_request(weight_buffers, gradient16_buffers, momentum_buffers, variance_buffers,
+                                        weight16_buffers, num_weights, buffer_sizes);
     if (int rc = prepare(device, req, -6, l, lock)) return rc;
     if (l.ctx != amp->ctx) {
         set_error("the loss-scale state belongs to another device context");
         return -16;
     }
-
-    StepParams p = zero_params();
-    p.lr = learning_rate;
-    p.beta1 = beta1;
-    p.beta2 = beta2;
-    p.one_minus_beta1 = 1.0f - beta1;
-    p.one_minus_beta2 = 1.0f - beta2;
-    p.eps = epsilon;
-    p.weight_decay = weight_decay;
-
-    // The context lock is held from here on: the issue counters of the loss-scale state are
-    // only read and advanced under it.  An asynchronous step's post-state goes into the ring
-    // slot of its issue number, a synchronous step's into slot 0.
-    AmpDeviceState *host_mirror = amp->h_pinned;
-    AmpBiasTable bias{};
-    if (async) {
-        if (!amp_poll(amp, true)) return -6;
-        host_mirror = &amp->h_pinned[1 + (amp->issued + 1) % kAmpMaxInFlight];
-        const int in_flight = (int)(amp->issued - amp->confirmed_issue);
-        if (in_flight > amp->max_in_flight) amp->max_in_flight = in_flight;
-        bias.base = amp->confirmed_applied;
-        bias.count = in_flight + 1;
-        for (int j = 0; j <= in_flight; j++)
-            gm_bias_corrections(beta1, beta2, amp->confirmed_applied + 1 + j, &bias.bc1[j], &bias.bc2[j]);
-    } else {
-        bias.count = 1;
-        gm_bias_corrections(beta1, beta2, step_count, &bias.bc1[0], &bias.bc2[0]);
-    }
+    const StepParams p = amp_step_params(learning_rate, beta1, beta2, epsilon, weight_decay);
+    AmpDeviceState *host_mirror;
+    AmpBiasTable bias;
+    if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
 
     const uint32_t chunks = l.plan->num_chunks;
     hipStream_t st = l.ctx->stream;
@@ -448,7 +590,86 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
 #undef GM_LAUNCH_AMP_B
 #undef GM_LAUNCH_AMP
     }
-    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror);
+    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror, 0);
+    return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
+}
+
+// The ping-pong step: one plan per set (identical geometry: same sizes, same planner), one fused
+// launch per segment, the epilogue, the repair pass.
+constexpr unsigned int kRepairGrid = 2048;
+static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const set_a[3], uintptr_t *const set_b[3],
+                             uintptr_t *gradient16_buffers, uintptr_t *weight16_buffers, int num_weights,
+                             int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
+                             float weight_decay, int step_count, bool async, Launch &l,
+                             std::unique_lock<std::mutex> &lock)
+{
+    for (int k = 0; k < 3; k++) {
+        if (num_weights > 0 && (!set_a[k] || !set_b[k])) {
+            set_error("both sets of weight, momentum and variance arrays are required");
+            return -4;
+        }
+    }
+    const PlanRequest req_a = amp_request(set_a[0], gradient16_buffers, set_a[1], set_a[2], weight16_buffers,
+                                          num_weights, buffer_sizes);
+    const PlanRequest req_b = amp_request(set_b[0], gradient16_buffers, set_b[1], set_b[2], weight16_buffers,
+                                          num_weights, buffer_sizes);
+    if (int rc = prepare(device, req_a, -6, l, lock)) return rc;
+    if (l.ctx != amp->ctx) {
+        set_error("the loss-scale state belongs to another device context");
+        return -16;
+    }
+    MultiTensorPlan *plan_a = l.plan;
+    // (the lock is held; the plan just found sits at the front of the cache and cannot be the one
+    // pushed out by the second lookup)
+    MultiTensorPlan *plan_b = get_plan(l.ctx, req_b);
+    if (!plan_b) return -6;
+    if (plan_b->status != 0) {
+        set_error("a required buffer handle of set B is nil (code %d)", plan_b->status);
+        return plan_b->status;
+    }
+    if (plan_a->num_chunks != plan_b->num_chunks || plan_a->num_segments != plan_b->num_segments ||
+        plan_a->segment[0].num_chunks != plan_b->segment[0].num_chunks ||
+        plan_a->segment[0].chunk_elements != plan_b->segment[0].chunk_elements ||
+        plan_a->segment[1].chunk_elements != plan_b->segment[1].chunk_elements ||
+        plan_a->total_elements != plan_b->total_elements) {
+        // only a tensor skipped in one set and not the other (a buffer shorter than its size) gets here
+        set_error("sets A and B do not hold the same tensors (a buffer of one set is shorter than its tensor)");
+        return -4;
+    }
+    const StepParams p = amp_step_params(learning_rate, beta1, beta2, epsilon, weight_decay);
+    AmpDeviceState *host_mirror;
+    AmpBiasTable bias;
+    if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
+
+    hipStream_t st = l.ctx->stream;
+    if (plan_a->num_chunks > 0) {
+        int vec = current_vec();
+        if (vec == 0) vec = auto_vec(8);
+        const bool nt = current_nontemporal();
+        int block = current_block();
+        if (block == 0) block = auto_block(8);
+        SegmentLaunch seg[2];
+        int count;
+        if (!launch_geometry(*plan_a, vec, block, seg, count)) return -6;
+#define GM_LAUNCH_FUSED(V, N, B) \
+        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, amp->d_state, bias)
+#define GM_LAUNCH_FUSED_B(B)                                                              \
+        if (vec == 4) { if (nt) GM_LAUNCH_FUSED(4, true, B); else GM_LAUNCH_FUSED(4, false, B); }        \
+        else if (vec == 2) { if (nt) GM_LAUNCH_FUSED(2, true, B); else GM_LAUNCH_FUSED(2, false, B); }   \
+        else { if (nt) GM_LAUNCH_FUSED(1, true, B); else GM_LAUNCH_FUSED(1, false, B); }
+        for (int s = 0; s < count; s++) {
+            const SegmentLaunch &g = seg[s];
+            if (block == 128) { GM_LAUNCH_FUSED_B(128) } else { GM_LAUNCH_FUSED_B(kBlock) }
+        }
+#undef GM_LAUNCH_FUSED_B
+#undef GM_LAUNCH_FUSED
+    }
+    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror, 1);
+    if (plan_a->num_chunks > 0 && weight16_buffers) {
+        const unsigned int grid = plan_a->num_chunks < kRepairGrid ? plan_a->num_chunks : kRepairGrid;
+        amp_repair_weight16_kernel<<<grid, kBlock, 0, st>>>(plan_a->d_chunks, plan_b->d_chunks, plan_a->num_chunks,
+                                                           amp->d_state);
+    }
     return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
 }
 
@@ -501,6 +722,79 @@ try {
     const int slot = (int)(issue % kAmpMaxInFlight);
     if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
         // the step itself is enqueued; resynchronise the bookkeeping with the device
+        (void)amp_download(amp);
+        return -6;
+    }
+    amp->issued = issue;
+    return 0;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int gm_amp_state_current_set(uintptr_t amp_state)
+try {
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    return s->h_pinned->current_set;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int execute_adam_amp_step_fused(uintptr_t device, uintptr_t *weight_a, uintptr_t *momentum_a, uintptr_t *variance_a,
+                                uintptr_t *weight_b, uintptr_t *momentum_b, uintptr_t *variance_b,
+                                uintptr_t *gradient16_buffers, uintptr_t *weight16_buffers, int num_weights,
+                                int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
+                                float weight_decay, int step_count, uintptr_t amp_state, int *skipped,
+                                float *scale_out, int *growth_tracker_out, int *current_set_out)
+try {
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    uintptr_t *const a[3] = {weight_a, momentum_a, variance_a};
+    uintptr_t *const b[3] = {weight_b, momentum_b, variance_b};
+    if (int rc = amp_enqueue_fused(device, amp, a, b, gradient16_buffers, weight16_buffers, num_weights, buffer_sizes,
+                                   learning_rate, beta1, beta2, epsilon, weight_decay, step_count, false, l, lock))
+        return rc;
+    if (!hip_ok(hipStreamSynchronize(l.ctx->stream), "hipStreamSynchronize")) return -6;
+    amp->confirmed_issue = amp->issued;
+    amp->confirmed_applied = amp->h_pinned->applied_steps;
+    if (skipped) *skipped = amp->h_pinned->last_skipped;
+    if (scale_out) *scale_out = amp->h_pinned->scale;
+    if (growth_tracker_out) *growth_tracker_out = amp->h_pinned->growth_tracker;
+    if (current_set_out) *current_set_out = amp->h_pinned->current_set;
+    return 0;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int execute_adam_amp_step_fused_async(uintptr_t device, uintptr_t *weight_a, uintptr_t *momentum_a,
+                                      uintptr_t *variance_a, uintptr_t *weight_b, uintptr_t *momentum_b,
+                                      uintptr_t *variance_b, uintptr_t *gradient16_buffers,
+                                      uintptr_t *weight16_buffers, int num_weights, int *buffer_sizes,
+                                      float learning_rate, float beta1, float beta2, float epsilon,
+                                      float weight_decay, uintptr_t amp_state)
+try {
+    if (device == 0) return -1;
+    AmpState *amp = amp_from_handle(amp_state);
+    if (!amp) return -16;
+    Launch l{};
+    std::unique_lock<std::mutex> lock;
+    uintptr_t *const a[3] = {weight_a, momentum_a, variance_a};
+    uintptr_t *const b[3] = {weight_b, momentum_b, variance_b};
+    if (int rc = amp_enqueue_fused(device, amp, a, b, gradient16_buffers, weight16_buffers, num_weights, buffer_sizes,
+                                   learning_rate, beta1, beta2, epsilon, weight_decay, 0, true, l, lock))
+        return rc;
+    const uint64_t issue = amp->issued + 1;
+    const int slot = (int)(issue % kAmpMaxInFlight);
+    if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
         (void)amp_download(amp);
         return -6;
     }

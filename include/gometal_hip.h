@@ -307,6 +307,41 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *weight_buffers,
                                 float beta1, float beta2, float epsilon, float weight_decay,
                                 uintptr_t amp_state);
 
+/* The mixed-precision Adam step in ONE pass over ping-pong state.  Weights, momentum and variance
+ * exist twice, as sets A and B of equal shape; one set is current (set A after
+ * gm_amp_state_create).  The step reads the current set and the fp16 gradients, checks the
+ * gradients as it reads them, and writes the OTHER set plus the fp16 weight copy; only if no
+ * gradient was +-inf or NaN does the written set become the current one.  A dropped step
+ * therefore leaves the current set untouched without any buffer having been read twice: 28 bytes
+ * move per parameter, against 30 for execute_adam_amp_step, which updates in place and must check
+ * every gradient before it may write anything.  Arithmetic, skip decision, loss-scale sequence and
+ * step counting are those of execute_adam_amp_step; the current set after any sequence of steps
+ * equals, bit for bit, what the in-place step leaves in its buffers.
+ *   - Which set is current: *current_set_out (0 = A, 1 = B) after the synchronous step,
+ *     gm_amp_state_current_set (which waits) at any time.  The other set holds scratch.
+ *   - weight16_buffers (may be NULL, entries may be 0) receives half(w') speculatively; after a
+ *     dropped step a repair pass rewrites it as half(current weights).  Callers keep the invariant
+ *     "the fp16 copy is half of the current weights" from the start (convert_tensor_type once
+ *     before the first step); with it a dropped step leaves the copy bit-identical as well.
+ *   - Both sets must hold every tensor (a buffer shorter than its tensor in one set only: -4).
+ * The _async form enqueues and returns, exactly as execute_adam_amp_step_async does.
+ * Codes as execute_adam_amp_step. */
+int execute_adam_amp_step_fused(uintptr_t device, uintptr_t *weight_a, uintptr_t *momentum_a, uintptr_t *variance_a,
+                                uintptr_t *weight_b, uintptr_t *momentum_b, uintptr_t *variance_b,
+                                uintptr_t *gradient16_buffers, uintptr_t *weight16_buffers, int num_weights,
+                                int *buffer_sizes, float learning_rate, float beta1, float beta2, float epsilon,
+                                float weight_decay, int step_count, uintptr_t amp_state, int *skipped,
+                                float *scale_out, int *growth_tracker_out, int *current_set_out);
+int execute_adam_amp_step_fused_async(uintptr_t device, uintptr_t *weight_a, uintptr_t *momentum_a,
+                                      uintptr_t *variance_a, uintptr_t *weight_b, uintptr_t *momentum_b,
+                                      uintptr_t *variance_b, uintptr_t *gradient16_buffers,
+                                      uintptr_t *weight16_buffers, int num_weights, int *buffer_sizes,
+                                      float learning_rate, float beta1, float beta2, float epsilon,
+                                      float weight_decay, uintptr_t amp_state);
+/* 0 when set A holds the current weights and moments of the ping-pong step, 1 when set B does.
+ * Waits for every step in flight.  -16: nil state; -6: HIP error. */
+int gm_amp_state_current_set(uintptr_t amp_state);
+
 /* execute_adam_step_mpsgraph for callers that cannot allocate.  No counterpart in the reference:
  * it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc.  Same arguments, arithmetic, update kernel and results as execute_adam_step_mpsgraph;

@@ -35,9 +35,10 @@ def dev():
     return d
 
 
-def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
+def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed, fused=False):
     """inject_at: {step index: (tensor, element, fp16 bits)}; checkpoints: step indices (0-based) after which
-    all buffers are compared."""
+    all buffers are compared.  fused: the one-pass ping-pong step (two sets of weights and moments on the device,
+    the fp16 copy kept as half of the current weights from the start) instead of the in-place step."""
     pkg, lib, D, o = load_package(), dev.lib, dev.handle, oracle()
     n, total = len(sizes), sum(sizes)
     offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
@@ -52,6 +53,13 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
     d_w16 = dev.alloc(2 * total, zero=True)
     arr = pkg.handle_array
     c_w, c_m, c_v = arr(d_w), arr(d_m), arr(d_v)
+    shadow = []
+    if fused:
+        shadow = [[dev.alloc(4 * s) for s in sizes] for _ in range(3)]
+        c_shadow = [arr(hs) for hs in shadow]
+        for k, a in enumerate(w_host):                 # invariant of the ping-pong step: fp16 copy = half(weights)
+            assert lib.convert_tensor_type(d_w[k], d_w16 + 2 * int(offsets[k]), pkg.int_array([sizes[k]]), 1, 0, 2, D) == 0
+    current = [0]
     c_g16 = arr([d_g16 + 2 * int(off) for off in offsets[:-1]])
     c_w16 = arr([d_w16 + 2 * int(off) for off in offsets[:-1]])
     bs = pkg.int_array([4 * s for s in sizes])
@@ -61,7 +69,8 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
     # ---- oracle side
     m_host = [np.zeros(s, np.float32) for s in sizes]
     v_host = [np.zeros(s, np.float32) for s in sizes]
-    w16_host = [np.zeros(s, np.uint16) for s in sizes]
+    w16_host = [a.astype(np.float16).view(np.uint16) if fused else np.zeros(s, np.uint16)
+                for a, s in zip(w_host, sizes)]
     st = o.amp_state(65536.0, 2.0, 0.5, 2000)
     g_buffers = [np.empty((2 * total + 3) // 4, np.uint32) for _ in range(2)]
     free_buffers, work = queue.Queue(), queue.Queue(maxsize=1)
@@ -97,7 +106,8 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
 
     def compare(context):
         drain()
-        for name_, dh, host in (("w", d_w, w_host), ("m", d_m, m_host), ("v", d_v, v_host)):
+        now = (d_w, d_m, d_v) if current[0] == 0 else tuple(shadow)
+        for name_, dh, host in (("w", now[0], w_host), ("m", now[1], m_host), ("v", now[2], v_host)):
             for k in range(n):
                 got = dev.to_numpy(dh[k], sizes[k])
                 assert np.array_equal(got.view(np.uint32), host[k].view(np.uint32)), (context, name_, k)
@@ -122,9 +132,18 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
             words = g_buffers[b].size
             assert lib.copy_metal_buffer_to_int32_array(d_g16, g_buffers[b].ctypes.data_as(ctypes.c_void_p), words) == 0
             skipped, sc, tracker = ctypes.c_int(-1), ctypes.c_float(0), ctypes.c_int(-1)
-            rc = lib.execute_adam_amp_step(D, c_w, c_g16, c_m, c_v, c_w16, n, bs, hyper["lr"], hyper["beta1"],
-                                           hyper["beta2"], hyper["eps"], hyper["weight_decay"], applied + 1, amp,
-                                           ctypes.byref(skipped), ctypes.byref(sc), ctypes.byref(tracker))
+            if fused:
+                cur = ctypes.c_int(-1)
+                rc = lib.execute_adam_amp_step_fused(D, c_w, c_m, c_v, c_shadow[0], c_shadow[1], c_shadow[2], c_g16, c_w16,
+                                                     n, bs, hyper["lr"], hyper["beta1"], hyper["beta2"], hyper["eps"],
+                                                     hyper["weight_decay"], applied + 1, amp, ctypes.byref(skipped),
+                                                     ctypes.byref(sc), ctypes.byref(tracker), ctypes.byref(cur))
+                current[0] ^= 0 if skipped.value else 1
+                assert cur.value == current[0], (k, cur.value, current[0])
+            else:
+                rc = lib.execute_adam_amp_step(D, c_w, c_g16, c_m, c_v, c_w16, n, bs, hyper["lr"], hyper["beta1"],
+                                               hyper["beta2"], hyper["eps"], hyper["weight_decay"], applied + 1, amp,
+                                               ctypes.byref(skipped), ctypes.byref(sc), ctypes.byref(tracker))
             assert rc == 0, (rc, lib.gm_last_error())
             applied += 0 if skipped.value else 1
             scale = sc.value
@@ -144,7 +163,7 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed):
         work.put(None)
         worker.join(timeout=60)
         lib.gm_amp_state_destroy(amp)
-        for h in d_w + d_m + d_v + [d_g16, d_w16]:
+        for h in d_w + d_m + d_v + [d_g16, d_w16] + [x for hs in shadow for x in hs]:
             dev.free(h)
 
 
@@ -171,3 +190,27 @@ def test_config5_mixed_precision_full_size_20_steps(dev):
     inject = {6: (len(sizes) - 3, 1234, 0xFC00), 13: (2, 4096 * 11008 - 1, 0x7E00)}
     trace = run_schedule(dev, "config 5 mixed precision", sizes, hyper, 20, inject, {0, 9, 19}, seed=5)
     assert [t[0] for t in trace].count(1) == 2 and trace[-1][1] == 16384.0 and trace[-1][3] == 18
+
+
+def test_config4_full_size_one_pass_step_1500_steps(dev):
+    """The first 1500 steps of the same schedule through the one-pass ping-pong step."""
+    sizes = amp_125m_sizes()
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)
+    rng = np.random.default_rng(0x6D657461 + 4)
+    chosen = [int(k) for k in np.flatnonzero(rng.random(5000) < 0.005) if k < 1500]
+    inject = {}
+    for j, k in enumerate(chosen):
+        t = int(rng.integers(0, len(sizes)))
+        inject[k] = (t, int(rng.integers(0, sizes[t])), [0x7C00, 0xFC00, 0x7E00][j % 3])
+    assert len(inject) >= 5
+    trace = run_schedule(dev, "config 4, one pass", sizes, hyper, 1500, inject, {499, 999, 1499}, seed=4, fused=True)
+    assert trace[-1][3] == 1500 - len(inject)
+
+
+def test_config5_mixed_precision_full_size_one_pass_step_20_steps(dev):
+    sizes = transformer_block_sizes()
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)
+    inject = {0: (7, 5, 0x7C00), 6: (len(sizes) - 3, 1234, 0xFC00), 13: (2, 4096 * 11008 - 1, 0x7E00)}
+    trace = run_schedule(dev, "config 5 mixed precision, one pass", sizes, hyper, 20, inject, {0, 1, 9, 19}, seed=5,
+                         fused=True)
+    assert [t[0] for t in trace].count(1) == 3 and trace[-1][1] == 8192.0 and trace[-1][3] == 17

@@ -250,3 +250,59 @@ def test_guards_survive_the_mixed_precision_step(dev, chunk, vec, lanes):
         lib.gm_amp_state_destroy(amp)
         for s in streams.values():
             s.free()
+
+
+@pytest.mark.parametrize("chunk,vec,lanes", SHAPES)
+def test_guards_survive_the_one_pass_mixed_precision_step(dev, chunk, vec, lanes):
+    """The ping-pong step writes the set that is not current: guards around every tensor of BOTH sets and of
+    the two fp16 streams, over applied and dropped steps (so that each set is written at least twice)."""
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)
+    lib, o = dev.lib, oracle()
+    sizes = EDGE_SIZES
+    rng = np.random.default_rng(127)
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    m = [np.zeros(n, np.float32) for n in sizes]
+    v = [np.zeros(n, np.float32) for n in sizes]
+    w16 = [a.astype(np.float16).view(np.uint16) for a in w]
+    names = ("wa", "ma", "va", "wb", "mb", "vb")
+    streams = {k: Packed(dev, sizes, np.float32, fill=w if k == "wa" else None) for k in names}
+    streams["g16"] = Packed(dev, sizes, np.float16)
+    streams["w16"] = Packed(dev, sizes, np.float16, fill=w16)
+    c = {k: pkg.handle_array(s.views) for k, s in streams.items()}
+    bs = pkg.int_array([4 * n for n in sizes])
+    amp = lib.gm_amp_state_create(dev.handle, 65536.0, 2.0, 0.5, 2000)
+    st = o.amp_state()
+    assert amp
+    current = 0
+    try:
+        assert lib.gm_set_tuning(chunk, -1, vec) == 0
+        assert lib.gm_set_workgroup_lanes(lanes) == 0
+        for k_step in range(6):
+            g16 = [(rng.normal(0, 1e-4, n) * np.float32(st.scale)).astype(np.float16).view(np.uint16) for n in sizes]
+            if k_step in (1, 4):
+                g16[k_step][0] = 0x7E00
+            streams["g16"].upload(g16)
+            skipped, cur = ctypes.c_int(-1), ctypes.c_int(-1)
+            rc = lib.execute_adam_amp_step_fused(dev.handle, c["wa"], c["ma"], c["va"], c["wb"], c["mb"], c["vb"], c["g16"],
+                                                 c["w16"], len(sizes), bs, hyper["lr"], hyper["beta1"], hyper["beta2"],
+                                                 hyper["eps"], hyper["weight_decay"], int(st.step_count) + 1, amp,
+                                                 ctypes.byref(skipped), None, None, ctypes.byref(cur))
+            assert rc == 0, (rc, lib.gm_last_error())
+            want = o.adam_amp(w, g16, m, v, w16, state=st, **hyper)
+            current ^= 0 if want else 1
+            assert (skipped.value, cur.value) == (want, current) and want == (1 if k_step in (1, 4) else 0)
+        assert current == 0
+        for name, s in streams.items():
+            tensors, guards_ok = s.read()
+            assert guards_ok, f"one pass chunk={chunk} vec={vec} lanes={lanes}: stream {name} wrote into a guard at " \
+                              f"{s.bad_guards()}"
+            host = {"wa": w, "ma": m, "va": v, "w16": w16}.get(name)
+            if host is not None:
+                for i, (a, b) in enumerate(zip(tensors, host)):
+                    assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), (name, i, sizes[i])
+    finally:
+        assert lib.gm_set_tuning(0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(0) == 0
+        lib.gm_amp_state_destroy(amp)
+        for s in streams.values():
+            s.free()
