@@ -125,6 +125,8 @@ HOST_ABI = {
     "gmo_uses_pooling": (i, [u]),
     "gmo_set_log_progress": (None, [u, i]),
     "gmo_enable_mixed_precision": (i, [u, f, f, f, i]),
+    "gmo_enable_ping_pong": (i, [u]),
+    "gmo_current_set": (i, [u]),
     "gmo_step_amp": (i, [u, up, up, i, ip]),
     "gmo_step_amp_async": (i, [u, up, up, i]),
     "gmo_sync_amp": (i, [u, ctypes.POINTER(ctypes.c_uint64)]),
@@ -393,6 +395,12 @@ class HostOptimizer:
     def EnableMixedPrecision(self, initial_scale=65536.0, growth_factor=2.0, backoff_factor=0.5, growth_interval=2000):
         return self._err(self.lib.gmo_enable_mixed_precision(self.handle, initial_scale, growth_factor,
                                                              backoff_factor, growth_interval))
+
+    def EnablePingPong(self):
+        return self._err(self.lib.gmo_enable_ping_pong(self.handle))
+
+    def current_set(self):
+        return self.lib.gmo_current_set(self.handle)
 
     def GetStepCount(self):
         return self.lib.gmo_get_step_count(self.handle)

@@ -409,5 +409,62 @@ Error ExecuteAdamAMPStepAsync(Pointer device, const std::vector<Pointer> &weight
     return "";
 }
 
+static Error checkFusedLists(const std::vector<Pointer> setA[3], const std::vector<Pointer> setB[3],
+                             const std::vector<Pointer> &gradient16Buffers,
+                             const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes)
+{
+    const size_t n = setA[0].size();
+    for (int k = 0; k < 3; k++)
+        if (setA[k].size() != n || setB[k].size() != n) return Errorf("all buffer arrays must have the same length");
+    if (n != gradient16Buffers.size() || n != bufferSizes.size() ||
+        (!weight16Buffers.empty() && weight16Buffers.size() != n))
+        return Errorf("all buffer arrays must have the same length");
+    if (n == 0) return Errorf("%s", kEmptyList);
+    return "";
+}
+
+Error ExecuteAdamAMPStepFused(Pointer device, const std::vector<Pointer> setA[3], const std::vector<Pointer> setB[3],
+                              const std::vector<Pointer> &gradient16Buffers,
+                              const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes,
+                              float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
+                              int stepCount, Pointer ampState, bool *skipped, float *scale, int *growthTracker,
+                              int *currentSet)
+{
+    if (Error e = checkFusedLists(setA, setB, gradient16Buffers, weight16Buffers, bufferSizes); !e.empty()) return e;
+    const size_t n = setA[0].size();
+    auto wa = handles(setA[0], n), ma = handles(setA[1], n), va = handles(setA[2], n);
+    auto wb = handles(setB[0], n), mb = handles(setB[1], n), vb = handles(setB[2], n);
+    auto g = handles(gradient16Buffers, n), h = handles(weight16Buffers, n);
+    std::vector<int> sizes(bufferSizes);
+    int sk = 0;
+    int result = execute_adam_amp_step_fused(H(device), wa.data(), ma.data(), va.data(), wb.data(), mb.data(), vb.data(),
+                                             g.data(), weight16Buffers.empty() ? nullptr : h.data(), (int)n,
+                                             sizes.data(), learningRate, beta1, beta2, epsilon, weightDecay, stepCount,
+                                             H(ampState), &sk, scale, growthTracker, currentSet);
+    if (result != 0) return Errorf("Adam mixed-precision step failed with error code: %d", result);
+    if (skipped) *skipped = sk != 0;
+    return "";
+}
+
+Error ExecuteAdamAMPStepFusedAsync(Pointer device, const std::vector<Pointer> setA[3],
+                                   const std::vector<Pointer> setB[3], const std::vector<Pointer> &gradient16Buffers,
+                                   const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes,
+                                   float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
+                                   Pointer ampState)
+{
+    if (Error e = checkFusedLists(setA, setB, gradient16Buffers, weight16Buffers, bufferSizes); !e.empty()) return e;
+    const size_t n = setA[0].size();
+    auto wa = handles(setA[0], n), ma = handles(setA[1], n), va = handles(setA[2], n);
+    auto wb = handles(setB[0], n), mb = handles(setB[1], n), vb = handles(setB[2], n);
+    auto g = handles(gradient16Buffers, n), h = handles(weight16Buffers, n);
+    std::vector<int> sizes(bufferSizes);
+    int result = execute_adam_amp_step_fused_async(H(device), wa.data(), ma.data(), va.data(), wb.data(), mb.data(),
+                                                   vb.data(), g.data(), weight16Buffers.empty() ? nullptr : h.data(),
+                                                   (int)n, sizes.data(), learningRate, beta1, beta2, epsilon,
+                                                   weightDecay, H(ampState));
+    if (result != 0) return Errorf("Adam mixed-precision step failed with error code: %d", result);
+    return "";
+}
+
 }  // namespace cgo_bridge
 }  // namespace gometal

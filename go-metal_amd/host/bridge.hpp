@@ -118,5 +118,19 @@ Error ExecuteAdamAMPStepAsync(Pointer device, const std::vector<Pointer> &weight
                               float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
                               Pointer ampState);
 
+// The one-pass step over ping-pong state (execute_adam_amp_step_fused): set A / set B of weights,
+// momentum and variance; *currentSet (may be null) receives which set is current after the step.
+Error ExecuteAdamAMPStepFused(Pointer device, const std::vector<Pointer> setA[3], const std::vector<Pointer> setB[3],
+                              const std::vector<Pointer> &gradient16Buffers,
+                              const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes,
+                              float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
+                              int stepCount, Pointer ampState, bool *skipped, float *scale, int *growthTracker,
+                              int *currentSet);
+Error ExecuteAdamAMPStepFusedAsync(Pointer device, const std::vector<Pointer> setA[3],
+                                   const std::vector<Pointer> setB[3], const std::vector<Pointer> &gradient16Buffers,
+                                   const std::vector<Pointer> &weight16Buffers, const std::vector<int> &bufferSizes,
+                                   float learningRate, float beta1, float beta2, float epsilon, float weightDecay,
+                                   Pointer ampState);
+
 }  // namespace cgo_bridge
 }  // namespace gometal

@@ -464,8 +464,9 @@ try {
         break;
     case GMO_ADAM: {
         auto *o = static_cast<AdamOptimizerState *>(h->opt.get());
-        if (t == "momentum") v = &o->MomentumBuffers;
-        if (t == "variance") v = &o->VarianceBuffers;
+        if (t == "momentum") v = &o->CurrentMomentumBuffers();
+        if (t == "variance") v = &o->CurrentVarianceBuffers();
+        if (t == "weight") v = &o->CurrentWeightBuffers();       // ping-pong mode: where the fp32 weights are now
         break;
     }
     case GMO_RMSPROP: {
@@ -541,6 +542,31 @@ try {
     if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
     Error e = a->EnableMixedPrecision(initial_scale, growth_factor, backoff_factor, growth_interval);
     return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+int gmo_enable_ping_pong(uintptr_t opt)
+try {
+    if (!opt) return fail(Errorf("object handle is nil"));
+    auto *a = adam_of(opt);
+    if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
+    Error e = a->EnablePingPong();
+    return e.empty() ? ok() : fail(e);
+} catch (...) {
+    note_exception();
+    return -1;
+}
+
+int gmo_current_set(uintptr_t opt)
+try {
+    if (!opt) return fail(Errorf("object handle is nil"));
+    auto *a = adam_of(opt);
+    if (!a) return fail(Errorf("mixed precision is only available on the Adam optimizer"));
+    (void)a->CurrentWeightBuffers();          // brings the host's view up to date after asynchronous steps
+    ok();
+    return a->PingPong() ? a->currentSet : 0;
 } catch (...) {
     note_exception();
     return -1;

@@ -424,9 +424,10 @@ Error AdamOptimizerState::Step(const std::vector<Pointer> &gradientBuffers)
     StepCount++;
     ampCountDirty = true;
     // As in adam.go:191-227 the pooled entry point is not used even when a pool is set.
-    Error err = cgo_bridge::ExecuteAdamStepMPSGraph(device, WeightBuffers, gradientBuffers, MomentumBuffers,
-                                                    VarianceBuffers, bufferSizes, LearningRate, Beta1, Beta2,
-                                                    Epsilon, WeightDecay, (int)StepCount);
+    // (with ping-pong state the fp32 step updates whichever set is current, in place)
+    Error err = cgo_bridge::ExecuteAdamStepMPSGraph(device, CurrentWeightBuffers(), gradientBuffers,
+                                                    CurrentMomentumBuffers(), CurrentVarianceBuffers(), bufferSizes,
+                                                    LearningRate, Beta1, Beta2, Epsilon, WeightDecay, (int)StepCount);
     if (!err.empty()) return Errorf("Adam step execution failed: %s", err.c_str());
     return "";
 }
@@ -448,6 +449,58 @@ Error AdamOptimizerState::EnableMixedPrecision(float initialScale, float growthF
     return "";
 }
 
+Error AdamOptimizerState::EnablePingPong()
+{
+    if (ampState == nullptr) return Errorf("mixed precision is not enabled: call EnableMixedPrecision first");
+    if (pingPong) return "";
+    if (memoryManager == nullptr) return Errorf("memory manager cannot be nil");
+    for (Pointer w : WeightBuffers)
+        if (w == nullptr) return Errorf("weight buffers are not set: call SetWeightBuffers first");
+    std::vector<Pointer> *lists[3] = {&ShadowWeightBuffers, &ShadowMomentumBuffers, &ShadowVarianceBuffers};
+    for (auto *list : lists) {
+        list->assign(bufferSizes.size(), nullptr);
+        for (size_t i = 0; i < bufferSizes.size(); i++) {
+            (*list)[i] = memoryManager->AllocateBuffer(bufferSizes[i]);
+            if ((*list)[i] == nullptr) {
+                for (auto *undo : lists) {
+                    releaseAll(memoryManager, *undo);
+                    undo->clear();
+                }
+                return Errorf("failed to allocate ping-pong buffer for weight %d", (int)i);
+            }
+        }
+    }
+    pingPong = true;
+    currentSet = 0;
+    return "";
+}
+
+Error AdamOptimizerState::refreshCurrentSet()
+{
+    if (!pingPong) return "";
+    if (ampPending > 0)
+        if (Error e = SyncAMP(); !e.empty()) return e;
+    return "";
+}
+
+const std::vector<Pointer> &AdamOptimizerState::CurrentWeightBuffers()
+{
+    (void)refreshCurrentSet();
+    return pingPong && currentSet == 1 ? ShadowWeightBuffers : WeightBuffers;
+}
+
+const std::vector<Pointer> &AdamOptimizerState::CurrentMomentumBuffers()
+{
+    (void)refreshCurrentSet();
+    return pingPong && currentSet == 1 ? ShadowMomentumBuffers : MomentumBuffers;
+}
+
+const std::vector<Pointer> &AdamOptimizerState::CurrentVarianceBuffers()
+{
+    (void)refreshCurrentSet();
+    return pingPong && currentSet == 1 ? ShadowVarianceBuffers : VarianceBuffers;
+}
+
 Error AdamOptimizerState::SyncAMP(uint64_t *skippedSteps)
 {
     if (ampState == nullptr) return Errorf("mixed precision is not enabled: call EnableMixedPrecision first");
@@ -455,6 +508,11 @@ Error AdamOptimizerState::SyncAMP(uint64_t *skippedSteps)
     if (gm_amp_state_query(reinterpret_cast<uintptr_t>(ampState), &LossScale, &GrowthTracker, &applied, &skipped) != 0)
         return Errorf("failed to read loss-scale state: %s", gm_last_error());
     if (ampPending > 0) StepCount = (uint64_t)applied;     // the device counted the pending steps
+    if (pingPong) {
+        const int set = gm_amp_state_current_set(reinterpret_cast<uintptr_t>(ampState));
+        if (set < 0) return Errorf("failed to read the current ping-pong set: %s", gm_last_error());
+        currentSet = set;
+    }
     ampPending = 0;
     if (skippedSteps) *skippedSteps = (uint64_t)skipped;
     return "";
@@ -473,9 +531,17 @@ Error AdamOptimizerState::StepAMPAsync(const std::vector<Pointer> &gradient16Buf
             return Errorf("failed to set the device step count: %s", gm_last_error());
         ampCountDirty = false;
     }
-    Error err = cgo_bridge::ExecuteAdamAMPStepAsync(device, WeightBuffers, gradient16Buffers, MomentumBuffers,
-                                                    VarianceBuffers, weight16Buffers, bufferSizes, LearningRate,
-                                                    Beta1, Beta2, Epsilon, WeightDecay, ampState);
+    Error err;
+    if (pingPong) {
+        const std::vector<Pointer> a[3] = {WeightBuffers, MomentumBuffers, VarianceBuffers};
+        const std::vector<Pointer> b[3] = {ShadowWeightBuffers, ShadowMomentumBuffers, ShadowVarianceBuffers};
+        err = cgo_bridge::ExecuteAdamAMPStepFusedAsync(device, a, b, gradient16Buffers, weight16Buffers, bufferSizes,
+                                                       LearningRate, Beta1, Beta2, Epsilon, WeightDecay, ampState);
+    } else {
+        err = cgo_bridge::ExecuteAdamAMPStepAsync(device, WeightBuffers, gradient16Buffers, MomentumBuffers,
+                                                  VarianceBuffers, weight16Buffers, bufferSizes, LearningRate,
+                                                  Beta1, Beta2, Epsilon, WeightDecay, ampState);
+    }
     if (!err.empty()) return Errorf("Adam mixed-precision step execution failed: %s", err.c_str());
     ampPending++;
     return "";
@@ -498,10 +564,19 @@ std::pair<bool, Error> AdamOptimizerState::StepAMP(const std::vector<Pointer> &g
     }
     bool skipped = false;
     // StepCount advances only when the step is applied: the bias corrections are taken at StepCount + 1.
-    Error err = cgo_bridge::ExecuteAdamAMPStep(device, WeightBuffers, gradient16Buffers, MomentumBuffers,
-                                               VarianceBuffers, weight16Buffers, bufferSizes, LearningRate, Beta1,
-                                               Beta2, Epsilon, WeightDecay, (int)(StepCount + 1), ampState, &skipped,
-                                               &LossScale, &GrowthTracker);
+    Error err;
+    if (pingPong) {
+        const std::vector<Pointer> a[3] = {WeightBuffers, MomentumBuffers, VarianceBuffers};
+        const std::vector<Pointer> b[3] = {ShadowWeightBuffers, ShadowMomentumBuffers, ShadowVarianceBuffers};
+        err = cgo_bridge::ExecuteAdamAMPStepFused(device, a, b, gradient16Buffers, weight16Buffers, bufferSizes,
+                                                  LearningRate, Beta1, Beta2, Epsilon, WeightDecay, (int)(StepCount + 1),
+                                                  ampState, &skipped, &LossScale, &GrowthTracker, &currentSet);
+    } else {
+        err = cgo_bridge::ExecuteAdamAMPStep(device, WeightBuffers, gradient16Buffers, MomentumBuffers,
+                                             VarianceBuffers, weight16Buffers, bufferSizes, LearningRate, Beta1,
+                                             Beta2, Epsilon, WeightDecay, (int)(StepCount + 1), ampState, &skipped,
+                                             &LossScale, &GrowthTracker);
+    }
     if (!err.empty()) return {false, Errorf("Adam mixed-precision step execution failed: %s", err.c_str())};
     if (!skipped) StepCount++;
     return {skipped, ""};
@@ -525,9 +600,17 @@ void AdamOptimizerState::Cleanup()
     if (memoryManager != nullptr) {
         releaseAll(memoryManager, MomentumBuffers);
         releaseAll(memoryManager, VarianceBuffers);
+        releaseAll(memoryManager, ShadowWeightBuffers);
+        releaseAll(memoryManager, ShadowMomentumBuffers);
+        releaseAll(memoryManager, ShadowVarianceBuffers);
     }
     MomentumBuffers.clear();
     VarianceBuffers.clear();
+    ShadowWeightBuffers.clear();
+    ShadowMomentumBuffers.clear();
+    ShadowVarianceBuffers.clear();
+    pingPong = false;
+    currentSet = 0;
     WeightBuffers.clear();
     bufferSizes.clear();
 }
@@ -537,9 +620,9 @@ StateResult AdamOptimizerState::GetState()
     if (ampPending > 0)
         if (Error e = SyncAMP(); !e.empty()) return {nullptr, e};
     auto st = std::make_unique<OptimizerState>();
-    if (Error e = readBuffers(MomentumBuffers, bufferSizes, "momentum", "momentum", "momentum", st->StateData); !e.empty())
+    if (Error e = readBuffers(CurrentMomentumBuffers(), bufferSizes, "momentum", "momentum", "momentum", st->StateData); !e.empty())
         return {nullptr, e};
-    if (Error e = readBuffers(VarianceBuffers, bufferSizes, "variance", "variance", "variance", st->StateData); !e.empty())
+    if (Error e = readBuffers(CurrentVarianceBuffers(), bufferSizes, "variance", "variance", "variance", st->StateData); !e.empty())
         return {nullptr, e};
     st->Type = "Adam";
     st->Parameters = {{"learning_rate", LearningRate}, {"beta1", Beta1},
@@ -578,8 +661,8 @@ Error AdamOptimizerState::LoadState(const OptimizerState *state)
         int idx;
         if (Error e = checkTensor(tensor, bufferSizes, idx); !e.empty()) return e;
         Error e;
-        if (tensor.StateType == "momentum") e = writeBuffer(MomentumBuffers[idx], tensor, idx, "momentum");
-        else if (tensor.StateType == "variance") e = writeBuffer(VarianceBuffers[idx], tensor, idx, "variance");
+        if (tensor.StateType == "momentum") e = writeBuffer(CurrentMomentumBuffers()[idx], tensor, idx, "momentum");
+        else if (tensor.StateType == "variance") e = writeBuffer(CurrentVarianceBuffers()[idx], tensor, idx, "variance");
         else e = Errorf("unknown state type: %s", tensor.StateType.c_str());
         if (!e.empty()) return e;
     }

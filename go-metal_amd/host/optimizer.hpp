@@ -168,6 +168,18 @@ public:
     // Waits for the pending steps; *skippedSteps (may be null) receives how many steps have
     // been dropped since EnableMixedPrecision.
     Error SyncAMP(uint64_t *skippedSteps = nullptr);
+    // Switches StepAMP / StepAMPAsync to the one-pass step over ping-pong state: a second set of weight,
+    // momentum and variance buffers is taken from the memory manager, and every applied step makes the set it
+    // wrote the current one.  Call after SetWeightBuffers and EnableMixedPrecision.  From then on the weights
+    // live in CurrentWeightBuffers() (the caller's own buffers after an even number of applied steps, the
+    // shadow set after an odd number); GetState / LoadState read and write the current moments; the fp16
+    // weight copy passed to StepAMP must start out as half of the weights (ConvertTo(Float16)).
+    Error EnablePingPong();
+    bool PingPong() const { return pingPong; }
+    // The buffers holding the current fp32 weights / moments (waits for pending asynchronous steps).
+    const std::vector<Pointer> &CurrentWeightBuffers();
+    const std::vector<Pointer> &CurrentMomentumBuffers();
+    const std::vector<Pointer> &CurrentVarianceBuffers();
     float LossScale = 0.0f;     // as of the last StepAMP / SyncAMP / EnableMixedPrecision / LoadState
     int GrowthTracker = 0;
 
@@ -179,6 +191,12 @@ public:
     Pointer ampState = nullptr;
     int ampPending = 0;            // asynchronous steps issued since the last SyncAMP
     bool ampCountDirty = false;    // StepCount changed on the host since the device last saw it
+    bool pingPong = false;
+    int currentSet = 0;            // 0: WeightBuffers / MomentumBuffers / VarianceBuffers are current, 1: the shadows
+    std::vector<Pointer> ShadowWeightBuffers, ShadowMomentumBuffers, ShadowVarianceBuffers;
+
+private:
+    Error refreshCurrentSet();     // after asynchronous steps: asks the device which set is current
 };
 std::pair<std::unique_ptr<AdamOptimizerState>, Error> NewAdamOptimizer(const AdamConfig &config,
                                                                        const Shapes &weightShapes,

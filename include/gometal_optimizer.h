@@ -78,7 +78,8 @@ int      gmo_load_checkpoint_json(uintptr_t opt, const char *json);
  * as 0 / 1); NaN if the optimizer has no such field. */
 float     gmo_get_field(uintptr_t opt, const char *name);
 /* Handle of state buffer `index` of one kind: "momentum", "variance", "squared_grad_avg",
- * "gradient_avg", "squared_update_avg"; 0 if absent. */
+ * "gradient_avg", "squared_update_avg"; 0 if absent.  Adam also answers "weight" (the buffer that
+ * holds the current fp32 weights: the caller's own unless the ping-pong step has made the shadow set current). */
 uintptr_t gmo_state_buffer(uintptr_t opt, const char *state_type, int index);
 int       gmo_uses_pooling(uintptr_t opt);
 void      gmo_set_log_progress(uintptr_t opt, int on);               /* AdaGrad / AdaDelta print every 10 steps */
@@ -86,6 +87,12 @@ void      gmo_set_log_progress(uintptr_t opt, int on);               /* AdaGrad 
 /* Adam mixed precision (no counterpart in the reference's optimizer package) */
 int   gmo_enable_mixed_precision(uintptr_t adam, float initial_scale, float growth_factor, float backoff_factor,
                                  int growth_interval);
+/* EnablePingPong: StepAMP / StepAMPAsync become the one-pass step over two sets of weights and moments
+ * (execute_adam_amp_step_fused); call after SetWeightBuffers and EnableMixedPrecision.  The current fp32
+ * weights are then gmo_state_buffer(adam, "weight", i); gmo_current_set tells which set that is (0: the
+ * caller's buffers, 1: the shadow set; -1 on error). */
+int   gmo_enable_ping_pong(uintptr_t adam);
+int   gmo_current_set(uintptr_t adam);
 int   gmo_step_amp(uintptr_t adam, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers, int n,
                    int *skipped);
 int   gmo_step_amp_async(uintptr_t adam, const uintptr_t *gradient16_buffers, const uintptr_t *weight16_buffers,

@@ -136,6 +136,7 @@ int adam_like(uintptr_t device, uintptr_t *w, uintptr_t *g, uintptr_t *m, uintpt
 struct AmpState {
     float scale, growth, backoff;
     int interval, tracker, applied, skipped;
+    int current_set;
 };
 
 }  // namespace
@@ -388,7 +389,7 @@ int execute_lbfgs_step_mpsgraph_pooled(uintptr_t device, uintptr_t *w, uintptr_t
 uintptr_t gm_amp_state_create(uintptr_t device, float init_scale, float growth, float backoff, int interval)
 {
     if (device == 0) return 0;
-    return reinterpret_cast<uintptr_t>(new AmpState{init_scale, growth, backoff, interval, 0, 0, 0});
+    return reinterpret_cast<uintptr_t>(new AmpState{init_scale, growth, backoff, interval, 0, 0, 0, 0});
 }
 void gm_amp_state_destroy(uintptr_t h) { delete reinterpret_cast<AmpState *>(h); }
 
@@ -473,6 +474,71 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *w, uintptr_t *g16, 
 {
     return execute_adam_amp_step(device, w, g16, m, v, w16, n, sizes, lr, b1, b2, eps, wd, 0, amp, nullptr, nullptr,
                                  nullptr);
+}
+
+int gm_amp_state_current_set(uintptr_t h) { return h ? reinterpret_cast<AmpState *>(h)->current_set : -16; }
+
+// The one-pass step over ping-pong state: the current set is read, the other one written.
+int execute_adam_amp_step_fused(uintptr_t device, uintptr_t *wa, uintptr_t *ma, uintptr_t *va, uintptr_t *wb,
+                                uintptr_t *mb, uintptr_t *vb, uintptr_t *g16, uintptr_t *w16, int n, int *sizes, float,
+                                float, float, float, float, int, uintptr_t amp, int *skipped, float *scale_out,
+                                int *tracker_out, int *current_set_out)
+{
+    if (device == 0) return -1;
+    if (!amp) return -16;
+    if (!wa || !ma || !va || !wb || !mb || !vb) return -4;
+    AmpState *st = reinterpret_cast<AmpState *>(amp);
+    const bool b_current = st->current_set != 0;
+    uintptr_t *set_a[3] = {wa, ma, va}, *set_b[3] = {wb, mb, vb};
+    uintptr_t **in = b_current ? set_b : set_a;
+    uintptr_t **out = b_current ? set_a : set_b;
+    bool found = false;
+    for (int i = 0; i < n; i++) {
+        for (int k = 0; k < 3; k++)
+            if (!in[k][i] || !out[k][i]) return -4;
+        if (!g16 || !g16[i]) return -4;
+        const size_t numel = sizes[i] > 0 ? (size_t)sizes[i] / 4 : 0;
+        const uint16_t *g = reinterpret_cast<const uint16_t *>(g16[i]);
+        for (size_t e = 0; e < numel; e++) {
+            if ((g[e] & 0x7C00u) == 0x7C00u) found = true;
+            for (int k = 0; k < 3; k++)
+                reinterpret_cast<float *>(out[k][i])[e] = reinterpret_cast<const float *>(in[k][i])[e] + 1.0f;
+            if (w16 && w16[i]) reinterpret_cast<uint16_t *>(w16[i])[e] = f32_to_f16(reinterpret_cast<float *>(out[0][i])[e]);
+        }
+    }
+    if (found) {
+        const float next = st->scale * st->backoff;
+        if (next >= 1.17549435e-38f) st->scale = next;
+        st->tracker = 0;
+        st->skipped++;
+        for (int i = 0; i < n && w16; i++) {                    // the repair pass
+            if (!w16[i]) continue;
+            const size_t numel = sizes[i] > 0 ? (size_t)sizes[i] / 4 : 0;
+            for (size_t e = 0; e < numel; e++)
+                reinterpret_cast<uint16_t *>(w16[i])[e] = f32_to_f16(reinterpret_cast<float *>(in[0][i])[e]);
+        }
+    } else {
+        st->applied++;
+        st->current_set ^= 1;
+        if (++st->tracker == st->interval) {
+            const float next = st->scale * st->growth;
+            if (next <= 3.40282347e+38f) st->scale = next;
+            st->tracker = 0;
+        }
+    }
+    if (skipped) *skipped = found ? 1 : 0;
+    if (scale_out) *scale_out = st->scale;
+    if (tracker_out) *tracker_out = st->tracker;
+    if (current_set_out) *current_set_out = st->current_set;
+    return 0;
+}
+
+int execute_adam_amp_step_fused_async(uintptr_t device, uintptr_t *wa, uintptr_t *ma, uintptr_t *va, uintptr_t *wb,
+                                      uintptr_t *mb, uintptr_t *vb, uintptr_t *g16, uintptr_t *w16, int n, int *sizes,
+                                      float lr, float b1, float b2, float eps, float wd, uintptr_t amp)
+{
+    return execute_adam_amp_step_fused(device, wa, ma, va, wb, mb, vb, g16, w16, n, sizes, lr, b1, b2, eps, wd, 0, amp,
+                                       nullptr, nullptr, nullptr, nullptr);
 }
 
 int gm_synchronize(uintptr_t device) { return device ? 0 : -1; }

@@ -150,6 +150,22 @@ static void mixed_precision(uintptr_t device, uintptr_t mm)
     const std::string js = take(gmo_get_state_json(opt));
     CHECK(js.find("loss_scale") != std::string::npos);
     CHECK(gmo_load_state_json(opt, js.c_str()) == 0);
+
+    // the one-pass step over ping-pong state: clean gradients again
+    CHECK(zero_metal_buffer(device, g16[4], kSizes[4] * 2) == 0);
+    CHECK(gmo_current_set(opt) == 0);
+    CHECK(gmo_enable_ping_pong(opt) == 0 && gmo_enable_ping_pong(opt) == 0);
+    const uint64_t before = gmo_get_step_count(opt);
+    CHECK(gmo_step_amp(opt, g16, w16, kTensors, &skipped) == 0 && skipped == 0 && gmo_current_set(opt) == 1);
+    CHECK(gmo_state_buffer(opt, "weight", 0) != w[0] && gmo_state_buffer(opt, "weight", 0) != 0);
+    CHECK(gmo_step_amp_async(opt, g16, w16, kTensors) == 0);
+    CHECK(gmo_current_set(opt) == 0 && gmo_state_buffer(opt, "weight", 0) == w[0]);
+    CHECK(gmo_get_step_count(opt) == before + 2);
+    CHECK(copy_int32_array_to_metal_buffer(g16[4], words.data(), (int)words.size()) == 0);      // the inf again
+    CHECK(gmo_step_amp(opt, g16, w16, kTensors, &skipped) == 0 && skipped == 1 && gmo_current_set(opt) == 0);
+    const std::string js2 = take(gmo_get_state_json(opt));
+    CHECK(!js2.empty() && gmo_load_state_json(opt, js2.c_str()) == 0);
+    CHECK(gmo_step(opt, w, kTensors) == 0);                      // an fp32 step on the current set
     gmo_cleanup(opt);
     gmo_optimizer_free(opt);
     for (int i = 0; i < kTensors; i++) {

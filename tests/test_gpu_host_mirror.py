@@ -289,3 +289,99 @@ def test_step_amp_async_through_the_mirror(env):
     opt.free()
     for h in dw + dw16 + dg + dg32:
         dev.free(h)
+
+
+def test_ping_pong_mixed_precision_through_the_mirror(env):
+    """EnablePingPong: StepAMP / StepAMPAsync run the one-pass step over two sets of weights and moments.  The
+    current weights (state_buffer "weight"), the moments GetState reads, the fp16 copy and every counter follow
+    the oracle through synchronous steps, dropped steps, asynchronous steps, a plain fp32 step and a checkpoint
+    round trip into a second ping-pong optimizer; Cleanup returns the shadow buffers to the pool."""
+    dev, mm = env
+    rng = np.random.default_rng(19)
+    sizes = [int(np.prod(s)) for s in SHAPES]
+    cfg, hyper = CASES[2][1], CASES[2][2]
+    opt = make(env, "adam", cfg)
+    w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    dw = [dev.from_numpy(a) for a in w]
+    w16 = [a.astype(np.float16).view(np.uint16) for a in w]
+    dw16 = [dev.from_numpy(h) for h in w16]                      # the fp16 copy starts as half of the weights
+    dg = [dev.alloc(2 * n + 2) for n in sizes]
+    dg32 = [dev.alloc(4 * n) for n in sizes]
+    assert opt.EnablePingPong() == "mixed precision is not enabled: call EnableMixedPrecision first"
+    assert opt.SetWeightBuffers(dw) is None
+    assert opt.EnableMixedPrecision(4096.0, 2.0, 0.5, 3) is None
+    tier = dev.lib.gmo_find_pool_size(mm, 4 * sizes[4])
+    before_alloc = pool_allocated(dev, mm, tier)
+    assert opt.EnablePingPong() is None and opt.current_set() == 0
+    m = [np.zeros(n, np.float32) for n in sizes]
+    v = [np.zeros(n, np.float32) for n in sizes]
+    st = oracle().amp_state(4096.0, 2.0, 0.5, 3)
+
+    def grads(inject):
+        g16 = [(rng.normal(0, 1e-4, n) * st.scale).astype(np.float16).view(np.uint16) for n in sizes]
+        if inject:
+            g16[4][100] = 0x7C00
+        for h, g in zip(dg, g16):
+            dev.upload(h, g)
+        return g16
+
+    def check(o, context):
+        for k, n in enumerate(sizes):
+            assert np.array_equal(dev.to_numpy(o.state_buffer("weight", k), n).view(np.uint32), w[k].view(np.uint32)), (context, k)
+            assert np.array_equal(dev.to_numpy(o.state_buffer("momentum", k), n).view(np.uint32), m[k].view(np.uint32)), (context, k)
+            assert np.array_equal(dev.to_numpy(o.state_buffer("variance", k), n).view(np.uint32), v[k].view(np.uint32)), (context, k)
+            assert np.array_equal(dev.to_numpy(dw16[k], n, np.uint16), w16[k]), (context, k)
+
+    applied = 0
+    for k in range(6):                                           # synchronous steps, two of them dropped
+        g16 = grads(k in (0, 3))
+        skipped, err = opt.StepAMP(dg, dw16)
+        assert err is None
+        want = oracle().adam_amp(w, g16, m, v, w16, state=st, **hyper)
+        applied += 0 if want else 1
+        assert skipped == bool(want) and opt.current_set() == applied % 2
+        assert opt.GetStepCount() == st.step_count
+    check(opt, "synchronous")
+    assert (opt.state_buffer("weight", 0) == dw[0]) == (applied % 2 == 0)     # the caller's own buffers or the shadows
+    for k in range(5):                                           # asynchronous steps, one dropped
+        g16 = grads(k == 2)
+        assert opt.StepAMPAsync(dg, dw16) is None
+        want = oracle().adam_amp(w, g16, m, v, w16, state=st, **hyper)
+        applied += 0 if want else 1
+        dev.synchronize()                                        # (the gradient buffers are reused)
+    assert opt.current_set() == applied % 2 and opt.GetStepCount() == st.step_count
+    check(opt, "asynchronous")
+    # a plain fp32 step updates the current set in place
+    g = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
+    for h, a in zip(dg32, g):
+        dev.upload(h, a)
+    assert opt.Step(dg32) is None
+    for k in range(len(sizes)):
+        oracle().adam(w[k], g[k], m[k], v[k], step=int(st.step_count) + 1, **hyper)
+    st.step_count += 1
+    for k, n in enumerate(sizes):
+        assert np.array_equal(dev.to_numpy(opt.state_buffer("weight", k), n).view(np.uint32), w[k].view(np.uint32))
+    # checkpoint into a second ping-pong optimizer whose current set is its own set A
+    text, err = opt.GetStateJSON()
+    assert err is None
+    resumed = make(env, "adam", cfg)
+    dw2 = [dev.from_numpy(a) for a in w]
+    assert resumed.SetWeightBuffers(dw2) is None
+    assert resumed.EnableMixedPrecision(4096.0, 2.0, 0.5, 3) is None and resumed.EnablePingPong() is None
+    assert resumed.LoadStateJSON(text) is None
+    for h, a in zip(dw16, w):                                    # the fp16 copy of the restored weights
+        dev.upload(h, a.astype(np.float16).view(np.uint16))
+    w16 = [a.astype(np.float16).view(np.uint16) for a in w]
+    for k in range(3):
+        g16 = grads(k == 1)
+        skipped, err = resumed.StepAMP(dg, dw16)
+        assert err is None
+        assert skipped == bool(oracle().adam_amp(w, g16, m, v, w16, state=st, **hyper))
+    assert resumed.GetStepCount() == st.step_count
+    check(resumed, "resumed")
+    for o in (opt, resumed):
+        o.Cleanup()
+        o.free()
+    assert pool_allocated(dev, mm, tier)[0] >= before_alloc[0] + 2      # shadow buffers of that tier are back in the pool
+    for h in dw + dw2 + dw16 + dg + dg32:
+        dev.free(h)
