@@ -563,6 +563,11 @@ def main():
                      "copy_kernel_gbs": copy_gbs,
                      "frac_of_copy_kernel": achieved / copy_gbs},
     }
+    footprint = params * 4 * (2 + nstate)            # every stream of the step, in bytes
+    if footprint < 256 * 1024 * 1024:
+        result["roofline"]["note"] = (f"the step's {footprint / 1e6:.0f} MB stay in the 256 MB memory-side cache between "
+                                      "steps and the kernel is a few microseconds of launch latency: 'achieved' counts "
+                                      "algorithmic bytes per second, it is not an HBM figure for this workload")
 
     # ---- mixed-precision Adam on the same list (fp16 gradients, fp16 weight copy) ----
     if rule == "adam" and not args.no_amp:
