@@ -15,16 +15,24 @@
  *     rounds every node to binary32 by integer arithmetic, and a numpy
  *     float32 ufunc chain), on the inputs the reference's own bridge tests
  *     use (cgo_bridge/optimizer_test.go:54-59) plus edge values, and by
- *     closed forms / invariants in tests/test_oracle_properties.py.
+ *     closed forms / invariants in tests/test_oracle_properties.py, among
+ *     them checks that separate neighbouring formulas (epsilon inside or
+ *     outside the root, mu at t or t + 1, the old or the new E[dx^2], decay
+ *     into the update or into the gradient), each one shown to fail against
+ *     this file with the corresponding line changed.
  *     The reference's tests assert no numerical output for these functions
  *     (they only log), so the equations are pinned, not Apple's MPSGraph bits.
  *   - gm_oracle_f32_to_f16 / gm_oracle_f16_to_f32: pinned exhaustively
  *     against numpy's float16 casts (all 65536 half patterns, boundary set).
+ *     The bulk loops use inlined fast paths of both, equal to these functions
+ *     on every bit pattern (gm_oracle_f16_fast_mismatches over all 2^32 / 2^16).
  *   - gm_oracle_adam_amp_step: PARITY UNPINNED against the reference: the
  *     reference holds no implementation of loss scaling, only constants
  *     (training/model_trainer.go:258-270) and prose
  *     (docs/tutorials/mixed-precision.md:610-629).  The semantics are defined
- *     here and pinned by a pure-Python brute-force state machine.
+ *     here and pinned by a pure-Python brute-force state machine.  Its
+ *     applied-step loop has an eight-lane form for hosts with AVX2 + F16C,
+ *     held to the scalar loop bit for bit (gm_oracle_amp_vector_mismatches).
  */
 #ifndef GM_ORACLE_H
 #define GM_ORACLE_H
