@@ -146,30 +146,44 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     update_slice<AdamRule, VEC, NT, true, BLOCK>(ch, slice_shift, prm, inv_scale);
 }
 
-// The ping-pong step: one pass.  Reads weights and moments of the current set and the fp16
-// gradients, writes the other set and the fp16 weight copy, and raises the flag when a gradient
-// of its own is +-inf or NaN.  It never looks at the flag: what it writes becomes current only if
-// the epilogue finds the flag clear.
+// One lane's share in two halves, so that the kernel can issue its global loads, do its scalar
+// bookkeeping (bias-correction pick) while they are in flight, and only then compute and store.
+template <int N>
+struct FusedLoaded {
+    typename VecOf<float, N>::type W, M, V;
+    typename VecOf<unsigned short, N>::type H;
+};
+
 template <int N, bool NT>
-__device__ inline bool amp_fused_group(const Chunk &in, const Chunk &out, uint32_t first, const StepParams &prm,
-                                       float inv_scale)
+__device__ inline FusedLoaded<N> amp_fused_load(const Chunk &in, uint32_t first)
 {
     typedef typename VecOf<float, N>::type FV;
     typedef typename VecOf<unsigned short, N>::type UV;
+    FusedLoaded<N> x;
+    x.W = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotWeight]) + first));
+    x.H = stream_load<NT>(reinterpret_cast<const UV *>(reinterpret_cast<const unsigned short *>(in.p[kSlotGrad]) + first));
+    x.M = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotState0]) + first));
+    x.V = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotState1]) + first));
+    return x;
+}
+
+// Computes the update of the loaded share and stores it into the other set (and the fp16 copy);
+// true when one of its gradients is +-inf or NaN.
+template <int N, bool NT>
+__device__ inline bool amp_fused_finish(const FusedLoaded<N> &x, const Chunk &out, uint32_t first, const StepParams &prm,
+                                        float inv_scale)
+{
+    typedef typename VecOf<float, N>::type FV;
     typedef typename VecOf<_Float16, N>::type HV;
-    const FV W = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotWeight]) + first));
-    const UV H = stream_load<NT>(reinterpret_cast<const UV *>(reinterpret_cast<const unsigned short *>(in.p[kSlotGrad]) + first));
-    const FV M = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotState0]) + first));
-    const FV V = stream_load<NT>(reinterpret_cast<const FV *>(reinterpret_cast<const float *>(in.p[kSlotState1]) + first));
     FV Wn, Mn, Vn;
     HV Hn;
     bool bad = false;
 #pragma unroll
     for (int c = 0; c < N; c++) {
-        const unsigned short bits = lane_of<N>(H, c);
+        const unsigned short bits = lane_of<N>(x.H, c);
         bad |= (bits & 0x7C00u) == 0x7C00u;
-        float wv = lane_of<N>(W, c);
-        float sv[2] = {lane_of<N>(M, c), lane_of<N>(V, c)};
+        float wv = lane_of<N>(x.W, c);
+        float sv[2] = {lane_of<N>(x.M, c), lane_of<N>(x.V, c)};
         const float gv = (float)__builtin_bit_cast(_Float16, bits) * inv_scale;
         AdamRule::apply(wv, gv, sv, prm);
         set_lane<N>(Wn, c, wv);
@@ -185,22 +199,37 @@ __device__ inline bool amp_fused_group(const Chunk &in, const Chunk &out, uint32
     return bad;
 }
 
+// The ping-pong step: one pass.  Reads weights and moments of the current set and the fp16
+// gradients, writes the other set and the fp16 weight copy, and raises the flag when a gradient
+// of its own is +-inf or NaN.  It never looks at the flag: what it writes becomes current only if
+// the epilogue finds the flag clear.
+// (The state pointer is the first argument and the early exit tests the head: both make the
+// compiler fetch the state's head together with the two descriptors, straight after the kernel
+// arguments, instead of behind the first branch; that shortens the chain of dependent scalar
+// loads in front of the first global load from four to two.)
 template <int VEC, bool NT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
-amp_adam_fused_kernel(const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t slice_shift,
-                      StepParams prm, AmpDeviceState *__restrict__ state, AmpBiasTable bias)
+amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restrict__ set_a,
+                      const Chunk *__restrict__ set_b, uint32_t slice_shift, StepParams prm, AmpBiasTable bias)
 {
-    // three scalar loads issued together: the state's head and the chunk's descriptor in either set
     const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
     const uint32_t c = blockIdx.x >> slice_shift;
     const Chunk a = set_a[c];
     const Chunk b = set_b[c];
     const uint32_t slice = blockIdx.x & ((1u << slice_shift) - 1u);
-    if ((slice * BLOCK * VEC >= a.count) | (a.p[kSlotWeight] == nullptr) | (b.p[kSlotWeight] == nullptr)) return;
+    // (a reciprocal scale of zero bits cannot occur: the scale is finite)
+    if ((slice * BLOCK * VEC >= a.count) | (a.p[kSlotWeight] == nullptr) | (b.p[kSlotWeight] == nullptr) | (head.y == 0u))
+        return;
     const bool b_is_current = head.x != 0u;
     const Chunk &in = b_is_current ? b : a;
     const Chunk &out = b_is_current ? a : b;
     const float inv_scale = __uint_as_float(head.y);
+    // vec-wide lanes need both sets aligned for them
+    const LaneShare s = lane_share(a.count, a.flags & b.flags, slice, threadIdx.x, VEC, BLOCK);
+    const bool whole = s.count != 0 && (VEC == 1 || s.grouped);
+    FusedLoaded<VEC> loaded;
+    if (whole) loaded = amp_fused_load<VEC, NT>(in, s.first);
+
     const int applied = (int)head.w;
     int pick = bias.count > 1 ? applied - bias.base : 0;
     pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
@@ -214,15 +243,13 @@ amp_adam_fused_kernel(const Chunk *__restrict__ set_a, const Chunk *__restrict__
     }
     prm.bc1 = bc1;
     prm.bc2 = bc2;
-    // vec-wide lanes need both sets aligned for them
-    const LaneShare s = lane_share(a.count, a.flags & b.flags, slice, threadIdx.x, VEC, BLOCK);
+
     bool bad = false;
-    if (s.count != 0) {
-        if (VEC > 1 && s.grouped) {
-            bad = amp_fused_group<VEC, NT>(in, out, s.first, prm, inv_scale);
-        } else {
-            for (uint32_t e = 0; e < s.count; e++) bad |= amp_fused_group<1, NT>(in, out, s.first + e, prm, inv_scale);
-        }
+    if (whole) {
+        bad = amp_fused_finish<VEC, NT>(loaded, out, s.first, prm, inv_scale);
+    } else {
+        for (uint32_t e = 0; e < s.count; e++)
+            bad |= amp_fused_finish<1, NT>(amp_fused_load<1, NT>(in, s.first + e), out, s.first + e, prm, inv_scale);
     }
     // One atomic per wavefront that saw a hit, and none once the flag is up (a tensor of nothing but
     // inf would otherwise send millions of atomics to one address).
@@ -652,7 +679,7 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
         int count;
         if (!launch_geometry(*plan_a, vec, block, seg, count)) return -6;
 #define GM_LAUNCH_FUSED(V, N, B) \
-        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, amp->d_state, bias)
+        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(amp->d_state, g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, bias)
 #define GM_LAUNCH_FUSED_B(B)                                                              \
         if (vec == 4) { if (nt) GM_LAUNCH_FUSED(4, true, B); else GM_LAUNCH_FUSED(4, false, B); }        \
         else if (vec == 2) { if (nt) GM_LAUNCH_FUSED(2, true, B); else GM_LAUNCH_FUSED(2, false, B); }   \
