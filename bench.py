@@ -40,11 +40,14 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
 # file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
 MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10,
                         # the three launches of one mixed-precision step: check 2.026e9 + update 2.8345e10
-                        ("c5", "adam_amp"): 3.0371e10,
+                        ("c5", "adam_amp"): 3.0385e10,
+                        # the one-pass step over ping-pong state: a single update launch
+                        ("c5", "adam_amp_one_pass"): 2.8375e10,
                         # bytes per step, summed over the passes of a 10-pair step (profiles/lbfgs_c5_1b_hbm_traffic.md)
                         ("lbfgs-c5", 10): 352.68 * 1012301824}
 TRAFFIC_SOURCE = {("c5", "adam"): "profiles/adam_c5_1b_hbm_traffic.md",
                   ("c5", "adam_amp"): "profiles/adam_c5_1b_hbm_traffic.md",
+                  ("c5", "adam_amp_one_pass"): "profiles/adam_c5_1b_hbm_traffic.md",
                   ("lbfgs-c5", 10): "profiles/lbfgs_c5_1b_hbm_traffic.md"}
 
 
