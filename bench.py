@@ -474,13 +474,13 @@ def main():
     pkg = load_package()
     dev = pkg.Device()                 # raises if the library is not built or no GPU is visible
     lib, D = dev.lib, dev.handle
-    if lib.gm_set_tuning(args.chunk, args.nontemporal, args.vec) != 0:
+    if lib.gm_set_tuning(D, args.chunk, args.nontemporal, args.vec) != 0:
         sys.exit("invalid --chunk / --vec combination (a chunk is a power-of-two multiple of 256 * vec elements)")
-    if lib.gm_set_workgroup_lanes(args.lanes) != 0:
+    if lib.gm_set_workgroup_lanes(D, args.lanes) != 0:
         sys.exit("invalid --lanes (128 or 256)")
     if args.amp_check_order:
         nt_flag, rev_flag = (int(x) for x in args.amp_check_order.split(","))
-        lib.gm_set_amp_check_order(nt_flag, rev_flag)
+        lib.gm_set_amp_check_order(D, nt_flag, rev_flag)
 
     if args.workload in LBFGS_WORKLOADS:
         return bench_lbfgs(args, pkg, dev)

@@ -79,9 +79,9 @@ ABI = {
     "gm_fill_normal_f32": (i, [u, u, ctypes.c_size_t, ctypes.c_uint64, f, f]),
     "gm_fill_normal_f16": (i, [u, u, ctypes.c_size_t, ctypes.c_uint64, f, f, f]),
     "gm_copy_probe": (i, [u, u, u, ctypes.c_size_t]),
-    "gm_set_tuning": (i, [i, i, i]),
-    "gm_set_workgroup_lanes": (i, [i]),
-    "gm_set_amp_check_order": (i, [i, i]),
+    "gm_set_tuning": (i, [u, i, i, i]),
+    "gm_set_workgroup_lanes": (i, [u, i]),
+    "gm_set_amp_check_order": (i, [u, i, i]),
 }
 
 # name -> (restype, argtypes): every symbol include/gometal_optimizer.h declares

@@ -26,10 +26,6 @@ namespace gm {
 
 constexpr float kMinLossScale = 1.17549435e-38f;   // FLT_MIN
 constexpr float kMaxLossScale = 3.40282347e+38f;   // FLT_MAX
-// Measurement switches of the overflow check (gm_set_amp_check_order): cache policy of its loads
-// and the direction it walks the table in.
-static std::atomic<int> g_check_nontemporal{1};
-static std::atomic<int> g_check_reverse{0};
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 
 // Loss-scale state machine, resident in HBM next to the tensors.
@@ -397,10 +393,13 @@ static void amp_free(AmpState *s)
     delete s;
 }
 
-int gm_set_amp_check_order(int nontemporal, int reverse)
+int gm_set_amp_check_order(uintptr_t device, int nontemporal, int reverse)
 {
-    g_check_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
-    g_check_reverse.store(reverse < 0 ? 0 : (reverse ? 1 : 0));
+    if (device == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -2;
+    ctx->amp_check_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
+    ctx->amp_check_reverse.store(reverse < 0 ? 0 : (reverse ? 1 : 0));
     return 0;
 }
 
@@ -591,17 +590,17 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     const uint32_t chunks = l.plan->num_chunks;
     hipStream_t st = l.ctx->stream;
     if (chunks > 0) {
-        int vec = current_vec();
+        int vec = current_vec(l.ctx);
         if (vec == 0) vec = auto_vec(8);
-        const bool nt = current_nontemporal();
-        int block = current_block();
+        const bool nt = current_nontemporal(l.ctx);
+        int block = current_block(l.ctx);
         if (block == 0) block = auto_block(8);
         SegmentLaunch seg[2];
         int count;
         if (!launch_geometry(*l.plan, vec, block, seg, count)) return -6;
         // the check walks the whole table, one workgroup per chunk of either segment
-        const int reverse = g_check_reverse.load();
-        if (nt && g_check_nontemporal.load())
+        const int reverse = l.ctx->amp_check_reverse.load();
+        if (nt && l.ctx->amp_check_nontemporal.load())
             amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse);
         else
             amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse);
@@ -670,10 +669,10 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
 
     hipStream_t st = l.ctx->stream;
     if (plan_a->num_chunks > 0) {
-        int vec = current_vec();
+        int vec = current_vec(l.ctx);
         if (vec == 0) vec = auto_vec(8);
-        const bool nt = current_nontemporal();
-        int block = current_block();
+        const bool nt = current_nontemporal(l.ctx);
+        int block = current_block(l.ctx);
         if (block == 0) block = auto_block(8);
         SegmentLaunch seg[2];
         int count;

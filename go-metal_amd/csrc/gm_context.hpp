@@ -52,6 +52,14 @@ struct Context {
     std::atomic<uint64_t> plan_builds{0};             // chunk tables laid out so far (diagnostics)
     std::atomic<uint64_t> table_allocations{0};       // table slots allocated so far (diagnostics)
     void *noalloc_scratch = nullptr;                  // this GPU's address of the allocation-free step's table
+    // Launch-shape settings of this context (gm_set_tuning, gm_set_workgroup_lanes, gm_set_amp_check_order):
+    // measurement switches, every combination gives bit-identical results.
+    std::atomic<int> chunk_elements{0};               // elements per chunk; 0: chosen per plan
+    std::atomic<int> nontemporal{1};                  // streaming accesses carry the non-temporal hint
+    std::atomic<int> vec{0};                          // fp32 elements per lane; 0: chosen per launch
+    std::atomic<int> block{0};                        // lanes per workgroup of the update kernels; 0: chosen per launch
+    std::atomic<int> amp_check_nontemporal{1};        // cache policy of the in-place overflow check's loads
+    std::atomic<int> amp_check_reverse{0};            // the in-place overflow check walks the table backwards
     std::mutex stage_mu;                              // one staged copy at a time
     bool stage_ready = false;
     StageLane stage[kStageLanes];                     // created on first use, kept until the process ends

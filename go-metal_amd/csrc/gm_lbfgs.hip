@@ -47,7 +47,7 @@
 
 namespace gm {
 
-bool current_nontemporal();   // gm_plan_cache.hip
+bool current_nontemporal(const Context *ctx);   // gm_plan_cache.hip
 
 namespace {
 
@@ -598,7 +598,7 @@ void launch_dot(Context *ctx, const Plan &p, StreamArgs a, bool negate)
     const uint32_t grid = p.num_chunks << p.slice_shift;
     a.chunks = p.d_chunks;
     a.slice_shift = p.slice_shift;
-    const bool nt = current_nontemporal();
+    const bool nt = current_nontemporal(ctx);
     if (negate) {
         if (nt) lbfgs_dot_kernel<true, true><<<grid, kLanes, 0, ctx->stream>>>(a);
         else lbfgs_dot_kernel<true, false><<<grid, kLanes, 0, ctx->stream>>>(a);
@@ -615,7 +615,7 @@ void launch_stream(Context *ctx, const Plan &p, StreamArgs a)
     const uint32_t grid = p.num_chunks << p.slice_shift;
     a.chunks = p.d_chunks;
     a.slice_shift = p.slice_shift;
-    if (current_nontemporal()) lbfgs_stream_kernel<MODE, DOT, true><<<grid, kLanes, 0, ctx->stream>>>(a);
+    if (current_nontemporal(ctx)) lbfgs_stream_kernel<MODE, DOT, true><<<grid, kLanes, 0, ctx->stream>>>(a);
     else lbfgs_stream_kernel<MODE, DOT, false><<<grid, kLanes, 0, ctx->stream>>>(a);
 }
 
@@ -625,7 +625,7 @@ void launch_update(Context *ctx, const Plan &p, UpdateArgs a, bool from_gradient
     a.chunks = p.d_chunks;
     a.quarter_shift = p.slice_shift + 2;      // four 256-element workgroups to a 1024-element slice
     const uint32_t grid = p.num_chunks << a.quarter_shift;
-    const bool nt = current_nontemporal();
+    const bool nt = current_nontemporal(ctx);
     hipStream_t st = ctx->stream;
 #define GM_LAUNCH_UPDATE(F, Y)                                                        \
     do {                                                                              \

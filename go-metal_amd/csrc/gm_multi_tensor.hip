@@ -31,13 +31,13 @@ static int launch_rule(const Launch &l, const StepParams &prm, int hip_error_cod
 {
     if (l.plan->num_chunks == 0) return 0;
     constexpr int streams = 3 + 2 * Rule::NSTATE;          // w, g, states read; w, states written
-    int vec = current_vec(), block = current_block();
+    int vec = current_vec(l.ctx), block = current_block(l.ctx);
     if (vec == 0) vec = auto_vec(streams);
     if (block == 0) block = auto_block(streams);
     SegmentLaunch seg[2];
     int count;
     if (!launch_geometry(*l.plan, vec, block, seg, count)) return hip_error_code;
-    for (int s = 0; s < count; s++) launch_update<Rule>(l.ctx->stream, seg[s], prm, vec, block, current_nontemporal());
+    for (int s = 0; s < count; s++) launch_update<Rule>(l.ctx->stream, seg[s], prm, vec, block, current_nontemporal(l.ctx));
     return hip_ok(hipGetLastError(), "update kernel launch") ? 0 : hip_error_code;
 }
 
@@ -133,10 +133,10 @@ try {
     p.momentum = momentum;
     p.weight_decay = weight_decay;
     p.nesterov = nesterov;
-    int vec = current_vec();
+    int vec = current_vec(l.ctx);
     if (vec == 0) vec = auto_vec(5);
-    const bool nt = current_nontemporal();
-    int block = current_block();
+    const bool nt = current_nontemporal(l.ctx);
+    int block = current_block(l.ctx);
     // Without momentum every tensor takes the vanilla rule: two streams read, one written.  That mix
     // does best in single-wavefront workgroups (measured on MI355X: 8-byte lanes, 64 lanes per
     // workgroup 85-87 % of peak against 76-77 % in 128-lane workgroups).

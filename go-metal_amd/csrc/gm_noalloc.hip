@@ -129,7 +129,7 @@ try {
 
     // The list's chunk size, as the caching entry point chooses it for a single segment; if the
     // table would not fit, the next larger sizes are tried (more idle workgroups, same results).
-    int chunk = current_chunk_elements();
+    int chunk = current_chunk_elements(ctx);
     const bool chunk_forced = chunk != 0;
     if (!chunk_forced) chunk = choose_chunk_elements(req);
     uint64_t total_chunks = 0;
@@ -148,7 +148,7 @@ try {
     }
     if (total_chunks == 0) return 0;
 
-    int vec = current_vec(), block = current_block();
+    int vec = current_vec(ctx), block = current_block(ctx);
     if (vec == 0) vec = auto_vec(7);
     if (block == 0) block = auto_block(7);
     const PlanSegment segment{0, (uint32_t)total_chunks, chunk};
@@ -191,7 +191,7 @@ try {
     p.eps = epsilon;
     p.weight_decay = weight_decay;
     gm_bias_corrections(beta1, beta2, step_count, &p.bc1, &p.bc2);
-    launch_update<AdamRule>(st, launch, p, vec, block, current_nontemporal());
+    launch_update<AdamRule>(st, launch, p, vec, block, current_nontemporal(ctx));
     return hip_ok(hipGetLastError(), "allocation-free Adam launch") ? 0 : -6;
 } catch (...) {
     note_exception();

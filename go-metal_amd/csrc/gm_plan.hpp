@@ -47,13 +47,14 @@ MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req);
 // that do not touch the range stay valid.
 void plans_forget_range(Context *ctx, uintptr_t begin, size_t bytes);
 
+// The context's launch-shape settings.
 // Elements per chunk forced by the caller (tunable for sweeps); 0 = chosen per plan.
-int current_chunk_elements();
+int current_chunk_elements(const Context *ctx);
 // Whether streaming accesses carry the non-temporal hint.
-bool current_nontemporal();
+bool current_nontemporal(const Context *ctx);
 // fp32 elements per lane (1, 2 or 4); 0 = chosen per launch.
-int current_vec();
+int current_vec(const Context *ctx);
 // Lanes per workgroup of the update kernels; 0 = chosen per launch.
-int current_block();
+int current_block(const Context *ctx);
 
 }  // namespace gm

@@ -23,15 +23,10 @@ constexpr int kAutoFewStreams = 5;
 int auto_vec(int streams) { return streams <= kAutoFewStreams ? 2 : 1; }
 int auto_block(int streams) { return streams <= kAutoFewStreams ? 128 : 256; }
 
-static std::atomic<int> g_chunk_elements{0};   // 0: chosen per plan
-static std::atomic<int> g_nontemporal{1};
-static std::atomic<int> g_vec{0};               // 0: chosen per launch by auto_vec
-static std::atomic<int> g_block{0};             // lanes per workgroup of the update kernels; 0: auto_block
-
-int current_chunk_elements() { return g_chunk_elements.load(); }
-bool current_nontemporal() { return g_nontemporal.load() != 0; }
-int current_vec() { return g_vec.load(); }
-int current_block() { return g_block.load(); }
+int current_chunk_elements(const Context *ctx) { return ctx->chunk_elements.load(); }
+bool current_nontemporal(const Context *ctx) { return ctx->nontemporal.load() != 0; }
+int current_vec(const Context *ctx) { return ctx->vec.load(); }
+int current_block(const Context *ctx) { return ctx->block.load(); }
 
 StepParams zero_params()
 {
@@ -176,7 +171,7 @@ static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanReque
 
 MultiTensorPlan *get_plan(Context *ctx, const PlanRequest &req)
 {
-    const int chunk = current_chunk_elements();
+    const int chunk = current_chunk_elements(ctx);
     auto &plans = ctx->plans;
     for (size_t i = 0; i < plans.size(); i++) {
         if (plan_matches(*plans[i], req, chunk)) {
@@ -255,8 +250,11 @@ using namespace gm;
 
 extern "C" {
 
-int gm_set_tuning(int chunk_elements, int nontemporal, int vec)
+int gm_set_tuning(uintptr_t device, int chunk_elements, int nontemporal, int vec)
 {
+    if (device == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -2;
     const int v = vec == 0 ? 4 : vec;        // an automatic width may be 1 or 2: the chunk must suit both
     const int c = chunk_elements;
     if (vec != 0 && v != 1 && v != 2 && v != 4) return -1;
@@ -266,16 +264,19 @@ int gm_set_tuning(int chunk_elements, int nontemporal, int vec)
         const int slices = c / (256 * v);
         if ((slices & (slices - 1)) != 0) return -1;
     }
-    g_vec.store(vec);
-    g_chunk_elements.store(c);
-    g_nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
+    ctx->vec.store(vec);
+    ctx->chunk_elements.store(c);
+    ctx->nontemporal.store(nontemporal < 0 ? 1 : (nontemporal ? 1 : 0));
     return 0;
 }
 
-int gm_set_workgroup_lanes(int lanes)
+int gm_set_workgroup_lanes(uintptr_t device, int lanes)
 {
+    if (device == 0) return -1;
+    Context *ctx = resolve_device(device);
+    if (!ctx) return -2;
     if (lanes != 0 && lanes != 128 && lanes != 256) return -1;
-    g_block.store(lanes);
+    ctx->block.store(lanes);
     return 0;
 }
 

@@ -386,24 +386,26 @@ int gm_fill_normal_f16(uintptr_t device, uintptr_t buffer, size_t num_elements, 
  * kernels are compared with, and the known-size launch that calibrates the
  * profiler's FETCH_SIZE / WRITE_SIZE counters. */
 int gm_copy_probe(uintptr_t device, uintptr_t dst_buffer, uintptr_t src_buffer, size_t bytes);
-/* Launch-shape overrides for sweeps: elements per chunk (a power-of-two multiple of
+/* Launch-shape overrides for sweeps.  They belong to the device's context: every step issued on that
+ * device handle uses them from the next call on, steps on another context do not.  Elements per chunk (a power-of-two multiple of
  * 256 * vec, of 1024 when vec is automatic; 0 = default: 65536, 16384, 4096, 1024 or 256, the largest
  * that keeps idle workgroups under 5 % for the tensor list, plus a smaller size for the list's
  * small tensors when they would idle 16384 workgroups or more; a size given here applies to
  * the whole list), non-temporal memory hints
  * on/off (-1 = default on) and fp32 elements per lane (1, 2 or 4; 0 = default: 2 for rules
  * with up to five streams, else 1).
- * -1 if the combination is not valid (nothing changes). */
-int gm_set_tuning(int chunk_elements, int nontemporal, int vec);
+ * -1 if the combination is not valid or device is 0 (nothing changes), -2 without a usable GPU. */
+int gm_set_tuning(uintptr_t device, int chunk_elements, int nontemporal, int vec);
 /* Lanes per workgroup of the update kernels: 128 or 256; 0 = default (128 for rules with up to
- * five streams, else 256).  -1 on any other value (nothing changes). */
-int gm_set_workgroup_lanes(int lanes);
+ * five streams, else 256).  Per context, like gm_set_tuning.  -1 on any other value or device 0
+ * (nothing changes), -2 without a usable GPU. */
+int gm_set_workgroup_lanes(uintptr_t device, int lanes);
 
 /* The overflow check of the mixed-precision step, for re-measurement: whether its loads carry the
  * non-temporal hint (default 1; -1 = default) and whether it walks the chunk table backwards, ending
  * on the gradients the update pass reads first (default 0; -1 = default).  Results do not depend on
- * either.  Always 0. */
-int gm_set_amp_check_order(int nontemporal, int reverse);
+ * either.  Per context, like gm_set_tuning.  0, -1 for device 0, -2 without a usable GPU. */
+int gm_set_amp_check_order(uintptr_t device, int nontemporal, int reverse);
 
 #ifdef __cplusplus
 }

@@ -123,8 +123,8 @@ def test_launch_shape_variants_are_bit_identical(dev, chunk, nt, vec, lanes):
     rng = np.random.default_rng(5)
     sizes = [1, 2, 3, 5, 255, 257, 1023, 4097, 70001, 262147]
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
-    assert lib.gm_set_tuning(chunk, nt, vec) == 0
-    assert lib.gm_set_workgroup_lanes(lanes) == 0
+    assert lib.gm_set_tuning(dev.handle, chunk, nt, vec) == 0
+    assert lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
     try:
         for rule, hyper in (("adam", ADAM), ("sgd", dict(lr=0.01, momentum=0.9, weight_decay=0.0, nesterov=False)),
                             ("adadelta", dict(rho=0.9, eps=1e-6, weight_decay=0.0))):
@@ -153,11 +153,11 @@ def test_launch_shape_variants_are_bit_identical(dev, chunk, nt, vec, lanes):
         for h in parents.values():
             dev.free(h)
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0
-        assert lib.gm_set_workgroup_lanes(0) == 0
-    assert lib.gm_set_workgroup_lanes(64) == -1 and lib.gm_set_workgroup_lanes(192) == -1
-    assert lib.gm_set_tuning(1000, 1, 1) == -1 and lib.gm_set_tuning(0, 1, 3) == -1
-    assert lib.gm_set_tuning(768, 1, 1) == -1          # 3 slices: not a power of two
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
+    assert lib.gm_set_workgroup_lanes(dev.handle, 64) == -1 and lib.gm_set_workgroup_lanes(dev.handle, 192) == -1
+    assert lib.gm_set_tuning(dev.handle, 1000, 1, 1) == -1 and lib.gm_set_tuning(dev.handle, 0, 1, 3) == -1
+    assert lib.gm_set_tuning(dev.handle, 768, 1, 1) == -1          # 3 slices: not a power of two
 
 
 def test_two_threads_step_two_optimizers(dev):

@@ -249,8 +249,8 @@ def test_amp_launch_shape_variants_are_bit_identical(dev, vec, lanes):
     rng = np.random.default_rng(17)
     sizes = [1, 2, 3, 7, 255, 257, 1023, 4097, 70001]
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
-    assert lib.gm_set_tuning(0, -1, vec) == 0
-    assert lib.gm_set_workgroup_lanes(lanes) == 0
+    assert lib.gm_set_tuning(dev.handle, 0, -1, vec) == 0
+    assert lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
     try:
         pair = AmpPair(dev, w, dict(HYPER, weight_decay=1e-4), (1024.0, 2.0, 0.5, 3))
         try:
@@ -263,8 +263,8 @@ def test_amp_launch_shape_variants_are_bit_identical(dev, vec, lanes):
         finally:
             pair.close()
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0
-        assert lib.gm_set_workgroup_lanes(0) == 0
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
 
 
 def test_amp_over_many_tiny_tensors(dev):

@@ -116,7 +116,7 @@ def test_fused_step_in_every_launch_shape(dev, chunk, vec, lanes):
     rng = np.random.default_rng(61)
     sizes = [1, 2, 3, 7, 0, 255, 256, 257, 1023, 4097, 65536, 70001]
     w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
-    assert lib.gm_set_tuning(chunk, -1, vec) == 0 and lib.gm_set_workgroup_lanes(lanes) == 0
+    assert lib.gm_set_tuning(dev.handle, chunk, -1, vec) == 0 and lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
     try:
         pair = FusedPair(dev, w, HYPER, (1024.0, 2.0, 0.5, 3))
         try:
@@ -131,7 +131,7 @@ def test_fused_step_in_every_launch_shape(dev, chunk, vec, lanes):
         finally:
             pair.close()
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0 and lib.gm_set_workgroup_lanes(0) == 0
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0 and lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
 
 
 def test_fused_step_5000_step_schedule_at_reduced_size(dev):

@@ -151,13 +151,13 @@ def test_guards_survive_every_rule_in_every_launch_shape(dev, rule, hyper):
     lib = dev.lib
     try:
         for chunk, vec, lanes in SHAPES:
-            assert lib.gm_set_tuning(chunk, -1, vec) == 0, (chunk, vec)
-            assert lib.gm_set_workgroup_lanes(lanes) == 0
+            assert lib.gm_set_tuning(dev.handle, chunk, -1, vec) == 0, (chunk, vec)
+            assert lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
             run_guarded(dev, rule, hyper, EDGE_SIZES, steps=3, seed=101,
                         context=f"{rule} chunk={chunk} vec={vec} lanes={lanes}")
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0
-        assert lib.gm_set_workgroup_lanes(0) == 0
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
 
 
 def test_guards_survive_the_allocation_free_step(dev):
@@ -165,13 +165,13 @@ def test_guards_survive_the_allocation_free_step(dev):
     lib = dev.lib
     try:
         for chunk, vec, lanes in SHAPES:
-            assert lib.gm_set_tuning(chunk, -1, vec) == 0
-            assert lib.gm_set_workgroup_lanes(lanes) == 0
+            assert lib.gm_set_tuning(dev.handle, chunk, -1, vec) == 0
+            assert lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
             run_guarded(dev, "adam", hyper, EDGE_SIZES, steps=3, seed=103, fn=lib.execute_adam_step_noalloc,
                         context=f"noalloc chunk={chunk} vec={vec} lanes={lanes}")
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0
-        assert lib.gm_set_workgroup_lanes(0) == 0
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
 
 
 def test_guards_survive_a_two_segment_plan(dev):
@@ -222,8 +222,8 @@ def test_guards_survive_the_mixed_precision_step(dev, chunk, vec, lanes):
     st = o.amp_state()
     assert amp
     try:
-        assert lib.gm_set_tuning(chunk, -1, vec) == 0
-        assert lib.gm_set_workgroup_lanes(lanes) == 0
+        assert lib.gm_set_tuning(dev.handle, chunk, -1, vec) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
         for k_step in range(4):
             g16 = [(rng.normal(0, 1e-4, n) * 65536.0).astype(np.float16).view(np.uint16) for n in sizes]
             if k_step == 2:
@@ -245,8 +245,8 @@ def test_guards_survive_the_mixed_precision_step(dev, chunk, vec, lanes):
                 for i, (a, b) in enumerate(zip(tensors, host)):
                     assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), (name, i, sizes[i])
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0
-        assert lib.gm_set_workgroup_lanes(0) == 0
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
         lib.gm_amp_state_destroy(amp)
         for s in streams.values():
             s.free()
@@ -275,8 +275,8 @@ def test_guards_survive_the_one_pass_mixed_precision_step(dev, chunk, vec, lanes
     assert amp
     current = 0
     try:
-        assert lib.gm_set_tuning(chunk, -1, vec) == 0
-        assert lib.gm_set_workgroup_lanes(lanes) == 0
+        assert lib.gm_set_tuning(dev.handle, chunk, -1, vec) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, lanes) == 0
         for k_step in range(6):
             g16 = [(rng.normal(0, 1e-4, n) * np.float32(st.scale)).astype(np.float16).view(np.uint16) for n in sizes]
             if k_step in (1, 4):
@@ -301,8 +301,8 @@ def test_guards_survive_the_one_pass_mixed_precision_step(dev, chunk, vec, lanes
                 for i, (a, b) in enumerate(zip(tensors, host)):
                     assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), (name, i, sizes[i])
     finally:
-        assert lib.gm_set_tuning(0, -1, 0) == 0
-        assert lib.gm_set_workgroup_lanes(0) == 0
+        assert lib.gm_set_tuning(dev.handle, 0, -1, 0) == 0
+        assert lib.gm_set_workgroup_lanes(dev.handle, 0) == 0
         lib.gm_amp_state_destroy(amp)
         for s in streams.values():
             s.free()
