@@ -662,7 +662,7 @@ def main():
             "roofline": {"bound": "hbm", "achieved": fused_achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": fused_achieved / HBM_PEAK_GBS, "bytes_per_param": 28, "bytes_per_param_moved": 28,
                          **traffic_fields((args.workload, "adam_amp_one_pass")),
-                         "kernel": "amp_adam_fused_kernel + amp_finalize_kernel + amp_repair_weight16_kernel",
+                         "kernel": "amp_adam_fused_kernel + amp_finalize_repair_kernel",
                          "kernel_ms": fused_event,
                          "note": "weights and moments kept twice (ping-pong): the step reads the current set and "
                                  "writes the other, so a dropped step needs no second read of the gradients; each "

@@ -33,7 +33,9 @@ struct alignas(16) AmpDeviceState {
     // head: the 16 bytes every workgroup of the update kernel reads with one scalar load
     int current_set;        // ping-pong step: 0 = set A holds the current weights and moments, 1 = set B
     float inv_scale;        // 1.0f / scale, kept by whoever changes scale (IEEE division on host and device alike)
-    int found_inf;          // set by the check (or the fused update), consumed and cleared by the epilogue
+    unsigned int found_inf; // the stamp of the step whose gradients held an inf / NaN (every step carries its own
+                            // non-zero stamp, so the word needs no clearing between the kernels of a step: it means
+                            // "this step overflowed" only while it equals this step's stamp)
     int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
     // tail
     float scale;
@@ -63,7 +65,8 @@ struct AmpBiasTable {
 // one atomic per workgroup that saw a hit.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
-amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state, int reverse)
+amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state, int reverse,
+                          unsigned int stamp)
 {
     __shared__ unsigned int wave_hit[kBlock / 64];
     // reverse: the table is walked from its end, so that the check finishes on the gradients the
@@ -103,7 +106,7 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__re
         unsigned int any = 0;
 #pragma unroll
         for (int k = 0; k < kBlock / 64; k++) any |= wave_hit[k];
-        if (any) atomicOr(&state->found_inf, 1);
+        if (any) __hip_atomic_store(&state->found_inf, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -112,7 +115,7 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__re
 template <int VEC, bool NT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
-                       const AmpDeviceState *__restrict__ state, AmpBiasTable bias)
+                       const AmpDeviceState *__restrict__ state, AmpBiasTable bias, unsigned int stamp)
 {
     // The state's head (current set, reciprocal of the scale, flag, applied steps) comes with one 16-byte scalar load
     // and the chunk descriptor with another, both issued before anything is decided; the bias
@@ -123,7 +126,7 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
     // (the weight pointer is never null; testing it here makes the compiler fetch the whole
     // descriptor before the branch instead of the count first and the addresses after it)
-    if ((head.z != 0u) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
+    if ((head.z == stamp) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
         return;                                                        // step dropped, or an idle slice
     const float inv_scale = __uint_as_float(head.y);
     const int applied = (int)head.w;
@@ -206,7 +209,8 @@ __device__ inline bool amp_fused_finish(const FusedLoaded<N> &x, const Chunk &ou
 template <int VEC, bool NT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restrict__ set_a,
-                      const Chunk *__restrict__ set_b, uint32_t slice_shift, StepParams prm, AmpBiasTable bias)
+                      const Chunk *__restrict__ set_b, uint32_t slice_shift, StepParams prm, AmpBiasTable bias,
+                      unsigned int stamp)
 {
     const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
     const uint32_t c = blockIdx.x >> slice_shift;
@@ -247,43 +251,21 @@ amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restric
         for (uint32_t e = 0; e < s.count; e++)
             bad |= amp_fused_finish<1, NT>(amp_fused_load<1, NT>(in, s.first + e), out, s.first + e, prm, inv_scale);
     }
-    // One atomic per wavefront that saw a hit, and none once the flag is up (a tensor of nothing but
-    // inf would otherwise send millions of atomics to one address).
+    // One store per wavefront that saw a hit, and none once the stamp is in (a tensor of nothing but
+    // inf would otherwise send millions of stores to one address).  Every writer stores the same value.
     const unsigned long long hit = __ballot(bad);
     if (hit != 0ull && (threadIdx.x & 63u) == (unsigned int)(__ffsll((long long)hit) - 1) &&
-        __hip_atomic_load(&state->found_inf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
-        atomicOr(&state->found_inf, 1);
+        __hip_atomic_load(&state->found_inf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stamp)
+        __hip_atomic_store(&state->found_inf, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// After a dropped ping-pong step the fp16 weight copy holds what the discarded update wrote:
-// it is rewritten from the current weights (the copy of an applied step is half(w) by
-// construction, so this restores it bit for bit).  Launched after the epilogue of every
-// ping-pong step on a small fixed grid; after an applied step every workgroup returns on its
-// first load.
-__global__ void __launch_bounds__(kBlock)
-amp_repair_weight16_kernel(const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t num_chunks,
-                           const AmpDeviceState *__restrict__ state)
+// Advances the loss-scale state machine after a step (one lane).  found: this step's gradients held
+// an inf / NaN.  The stamp word is left alone while it names this step and zeroed otherwise, so a
+// stale stamp can never meet its own value again when the 32-bit stamp counter wraps.
+__device__ inline void amp_advance(AmpDeviceState *state, AmpDeviceState *host_mirror, bool found, unsigned int stamp,
+                                   int ping_pong)
 {
-    if (state->last_skipped == 0) return;
-    const Chunk *current = state->current_set != 0 ? set_b : set_a;
-    for (uint32_t c = blockIdx.x; c < num_chunks; c += gridDim.x) {
-        const Chunk ch = current[c];
-        if (ch.p[kSlotWeight16] == nullptr) continue;
-        const float *w = reinterpret_cast<const float *>(ch.p[kSlotWeight]);
-        _Float16 *h = reinterpret_cast<_Float16 *>(ch.p[kSlotWeight16]);
-        for (uint32_t e = threadIdx.x; e < ch.count; e += kBlock) h[e] = (_Float16)w[e];
-    }
-}
-
-// Epilogue (one lane, same stream, after phase B has drained): advances the
-// loss-scale state machine and re-arms the flag.  A separate launch rather
-// than a last-workgroup ticket: a single counter bumped by every workgroup of
-// a 250k-workgroup grid serialises in the memory-side atomic unit.
-__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror, int ping_pong)
-{
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
     AmpDeviceState st = *state;
-    const int found = st.found_inf;
     // The scale stays a normal, finite fp32 number whatever the run does: a growth that would
     // overflow to infinity (about 112 uninterrupted growth intervals from 65536) and a backoff
     // that would leave the normal range are not applied.  Unbounded, the scale would stick at
@@ -305,11 +287,45 @@ __global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_
     }
     st.inv_scale = 1.0f / st.scale;
     st.last_skipped = found ? 1 : 0;
-    st.found_inf = 0;
+    st.found_inf = found ? stamp : 0u;
     *state = st;
     // The post-state also goes straight into pinned host memory: the host reads it once the
     // stream (or the event recorded after this launch) has completed, without a copy launch.
     if (host_mirror) *host_mirror = st;
+}
+
+// Epilogue of the in-place step (one lane, same stream, after the update pass has drained).  A
+// separate launch rather than a last-workgroup ticket: a single counter bumped by every workgroup
+// of a 250k-workgroup grid serialises in the memory-side atomic unit.
+__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror, unsigned int stamp)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    amp_advance(state, host_mirror, state->found_inf == stamp, stamp, 0);
+}
+
+// Epilogue of the ping-pong step, and the repair of the fp16 weight copy, in one launch.  After a
+// dropped step the copy holds what the discarded update wrote: it is rewritten from the current
+// weights (the copy of an applied step is half(w) by construction, so this restores it bit for
+// bit).  Small fixed grid; after an applied step every workgroup returns on its first load.
+// Lane 0 of workgroup 0 advances the state machine while the other workgroups read two words of
+// the same record; that is safe because whatever those readers act on does not change under them:
+// the stamp word either keeps naming this step (dropped: they repair, and the current set is not
+// flipped) or goes from one value that is not this step's stamp to another (applied: they return).
+__global__ void __launch_bounds__(kBlock)
+amp_finalize_repair_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror, unsigned int stamp,
+                           const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t num_chunks)
+{
+    const bool found = __hip_atomic_load(&state->found_inf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == stamp;
+    if (blockIdx.x == 0 && threadIdx.x == 0) amp_advance(state, host_mirror, found, stamp, 1);
+    if (!found) return;
+    const Chunk *current = __hip_atomic_load(&state->current_set, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ? set_b : set_a;
+    for (uint32_t c = blockIdx.x; c < num_chunks; c += gridDim.x) {
+        const Chunk ch = current[c];
+        if (ch.p[kSlotWeight16] == nullptr) continue;
+        const float *w = reinterpret_cast<const float *>(ch.p[kSlotWeight]);
+        _Float16 *h = reinterpret_cast<_Float16 *>(ch.p[kSlotWeight16]);
+        for (uint32_t e = threadIdx.x; e < ch.count; e += kBlock) h[e] = (_Float16)w[e];
+    }
 }
 
 }  // namespace gm
@@ -330,6 +346,7 @@ struct AmpState {
     uint64_t confirmed_issue;            // newest step whose post-state the host has seen
     int confirmed_applied;               // the device's applied_steps after that step
     int max_in_flight;                   // deepest run-ahead seen (diagnostics)
+    unsigned int last_stamp;             // stamp of the newest step issued (either form); never 0
 };
 static const uint64_t kAmpMagic = 0x676D5F616D705F73ull;   // "gm_amp_s"
 
@@ -511,6 +528,13 @@ try {
     return -6;
 }
 
+// The next step's stamp (the context lock is held).
+static unsigned int amp_next_stamp(AmpState *amp)
+{
+    if (++amp->last_stamp == 0u) ++amp->last_stamp;
+    return amp->last_stamp;
+}
+
 static StepParams amp_step_params(float learning_rate, float beta1, float beta2, float epsilon, float weight_decay)
 {
     StepParams p = zero_params();
@@ -586,6 +610,7 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     AmpDeviceState *host_mirror;
     AmpBiasTable bias;
     if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
+    const unsigned int stamp = amp_next_stamp(amp);
 
     const uint32_t chunks = l.plan->num_chunks;
     hipStream_t st = l.ctx->stream;
@@ -601,10 +626,10 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
         // the check walks the whole table, one workgroup per chunk of either segment
         const int reverse = l.ctx->amp_check_reverse.load();
         if (nt && l.ctx->amp_check_nontemporal.load())
-            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse);
+            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse, stamp);
         else
-            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse);
-#define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, amp->d_state, bias)
+            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse, stamp);
+#define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, amp->d_state, bias, stamp)
 #define GM_LAUNCH_AMP_B(B)                                                              \
         if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true, B); else GM_LAUNCH_AMP(4, false, B); }        \
         else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true, B); else GM_LAUNCH_AMP(2, false, B); }   \
@@ -616,12 +641,12 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
 #undef GM_LAUNCH_AMP_B
 #undef GM_LAUNCH_AMP
     }
-    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror, 0);
+    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror, stamp);
     return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
 }
 
 // The ping-pong step: one plan per set (identical geometry: same sizes, same planner), one fused
-// launch per segment, the epilogue, the repair pass.
+// launch per segment, then the epilogue and the repair pass in one launch.
 constexpr unsigned int kRepairGrid = 2048;
 static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const set_a[3], uintptr_t *const set_b[3],
                              uintptr_t *gradient16_buffers, uintptr_t *weight16_buffers, int num_weights,
@@ -666,6 +691,7 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
     AmpDeviceState *host_mirror;
     AmpBiasTable bias;
     if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
+    const unsigned int stamp = amp_next_stamp(amp);
 
     hipStream_t st = l.ctx->stream;
     if (plan_a->num_chunks > 0) {
@@ -678,7 +704,7 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
         int count;
         if (!launch_geometry(*plan_a, vec, block, seg, count)) return -6;
 #define GM_LAUNCH_FUSED(V, N, B) \
-        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(amp->d_state, g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, bias)
+        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(amp->d_state, g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, bias, stamp)
 #define GM_LAUNCH_FUSED_B(B)                                                              \
         if (vec == 4) { if (nt) GM_LAUNCH_FUSED(4, true, B); else GM_LAUNCH_FUSED(4, false, B); }        \
         else if (vec == 2) { if (nt) GM_LAUNCH_FUSED(2, true, B); else GM_LAUNCH_FUSED(2, false, B); }   \
@@ -690,12 +716,11 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
 #undef GM_LAUNCH_FUSED_B
 #undef GM_LAUNCH_FUSED
     }
-    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror, 1);
-    if (plan_a->num_chunks > 0 && weight16_buffers) {
-        const unsigned int grid = plan_a->num_chunks < kRepairGrid ? plan_a->num_chunks : kRepairGrid;
-        amp_repair_weight16_kernel<<<grid, kBlock, 0, st>>>(plan_a->d_chunks, plan_b->d_chunks, plan_a->num_chunks,
-                                                           amp->d_state);
-    }
+    // without an fp16 copy there is nothing to repair: one workgroup, for the epilogue alone
+    const bool repair = plan_a->num_chunks > 0 && weight16_buffers;
+    const unsigned int grid = !repair ? 1u : (plan_a->num_chunks < kRepairGrid ? plan_a->num_chunks : kRepairGrid);
+    amp_finalize_repair_kernel<<<grid, kBlock, 0, st>>>(amp->d_state, host_mirror, stamp, plan_a->d_chunks,
+                                                       plan_b->d_chunks, repair ? plan_a->num_chunks : 0u);
     return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
 }
 

@@ -236,3 +236,42 @@ def test_fused_step_argument_errors(dev):
         lib.gm_amp_state_destroy(amp)
         for h in list(bufs.values()) + [g16, short]:
             dev.free(h)
+
+
+def test_in_place_and_one_pass_steps_share_one_loss_scale_state(dev):
+    """Both forms advance the same device state and tell an overflow by the same per-step stamp: alternated on one
+    list (the in-place step working on whichever set is current), with dropped steps next to each other, before
+    and after applied ones and across the change of form, the sequence is the oracle's and nothing of an earlier
+    step's overflow leaks into a later one."""
+    lib = dev.lib
+    rng = np.random.default_rng(77)
+    sizes = [1, 255, 4096, 70001]
+    pair = FusedPair(dev, [rng.standard_normal(s).astype(np.float32) for s in sizes], HYPER, (1024.0, 2.0, 0.5, 3))
+    poisoned = {1, 2, 5, 8, 9, 10, 14}
+    forms = "FFIIFIFFIIFIIFFIFI"           # F: one pass, I: in place
+    try:
+        for k, form in enumerate(forms):
+            g16 = scaled_g16(rng, sizes, pair.st.scale)
+            if k in poisoned:
+                t = k % len(sizes)
+                g16[t][(k * 37) % sizes[t]] = [0x7C00, 0xFC00, 0x7E00][k % 3]
+            if form == "F":
+                assert pair.step(g16) == (1 if k in poisoned else 0)
+            else:
+                for hd, g in zip(pair.g16, g16):
+                    dev.upload(hd, g)
+                cur = pair.c[pair.current]
+                skipped, scale, tracker = ctypes.c_int(-1), ctypes.c_float(0), ctypes.c_int(-1)
+                rc = lib.execute_adam_amp_step(dev.handle, cur["w"], pair.c_g16, cur["m"], cur["v"], pair.c_w16, pair.n,
+                                               pair.bs, HYPER["lr"], HYPER["beta1"], HYPER["beta2"], HYPER["eps"],
+                                               HYPER["weight_decay"], int(pair.st.step_count) + 1, pair.amp,
+                                               ctypes.byref(skipped), ctypes.byref(scale), ctypes.byref(tracker))
+                assert rc == 0, (rc, lib.gm_last_error())
+                want = oracle().adam_amp(pair.w, g16, pair.m, pair.v, pair.w16, state=pair.st, **HYPER)
+                assert (skipped.value, scale.value, tracker.value) == (want, float(np.float32(pair.st.scale)),
+                                                                        pair.st.growth_tracker), (k, form)
+                assert want == (1 if k in poisoned else 0)
+                assert lib.gm_amp_state_current_set(pair.amp) == pair.current      # an in-place step never flips it
+            pair.compare(f"step {k} ({form})")
+    finally:
+        pair.close()
