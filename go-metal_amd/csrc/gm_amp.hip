@@ -110,6 +110,17 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__re
     }
 }
 
+// The bias corrections of the step count the device has reached: entry (applied - base) of the
+// table, clamped; entry 0 when the table has one entry.
+__device__ inline void amp_pick_bias(StepParams &prm, const AmpBiasTable &bias, int applied)
+{
+    int pick = bias.count > 1 ? applied - bias.base : 0;
+    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
+    // (the table sits in the kernel-argument segment: an indexed scalar load, no copy to scratch)
+    prm.bc1 = bias.bc1[pick];
+    prm.bc2 = bias.bc2[pick];
+}
+
 // Phase B: the Adam update on unscaled gradients, skipped as a whole when the
 // flag is set.
 template <int VEC, bool NT, int BLOCK>
@@ -119,8 +130,7 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
 {
     // The state's head (current set, reciprocal of the scale, flag, applied steps) comes with one 16-byte scalar load
     // and the chunk descriptor with another, both issued before anything is decided; the bias
-    // table sits in the kernel arguments and its entry is picked by scalar selects.  No load
-    // waits for another except on the kernel-argument pointers themselves.
+    // table sits in the kernel arguments and its entry comes with an indexed scalar load.
     const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
     const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
@@ -129,19 +139,7 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     if ((head.z == stamp) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
         return;                                                        // step dropped, or an idle slice
     const float inv_scale = __uint_as_float(head.y);
-    const int applied = (int)head.w;
-    int pick = bias.count > 1 ? applied - bias.base : 0;
-    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
-    float bc1 = bias.bc1[0], bc2 = bias.bc2[0];
-#pragma unroll
-    for (int j = 1; j < kAmpMaxInFlight; j++) {
-        if (pick == j) {
-            bc1 = bias.bc1[j];
-            bc2 = bias.bc2[j];
-        }
-    }
-    prm.bc1 = bc1;
-    prm.bc2 = bc2;
+    amp_pick_bias(prm, bias, (int)head.w);
     update_slice<AdamRule, VEC, NT, true, BLOCK>(ch, slice_shift, prm, inv_scale);
 }
 
@@ -218,7 +216,11 @@ amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restric
     const Chunk b = set_b[c];
     const uint32_t slice = blockIdx.x & ((1u << slice_shift) - 1u);
     // (a reciprocal scale of zero bits cannot occur: the scale is finite)
-    if ((slice * BLOCK * VEC >= a.count) | (a.p[kSlotWeight] == nullptr) | (b.p[kSlotWeight] == nullptr) | (head.y == 0u))
+    // (an empty bias table cannot occur either; testing it here brings its size and base in together
+    // with the descriptors, so the pick below is a dozen scalar instructions and not another
+    // fetch-and-wait in front of the global loads)
+    if ((slice * BLOCK * VEC >= a.count) | (a.p[kSlotWeight] == nullptr) | (b.p[kSlotWeight] == nullptr) | (head.y == 0u) |
+        (bias.count < 1) | (bias.base < 0))
         return;
     const bool b_is_current = head.x != 0u;
     const Chunk &in = b_is_current ? b : a;
@@ -229,21 +231,7 @@ amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restric
     const bool whole = s.count != 0 && (VEC == 1 || s.grouped);
     FusedLoaded<VEC> loaded;
     if (whole) loaded = amp_fused_load<VEC, NT>(in, s.first);
-
-    const int applied = (int)head.w;
-    int pick = bias.count > 1 ? applied - bias.base : 0;
-    pick = pick < 0 ? 0 : (pick >= bias.count ? bias.count - 1 : pick);
-    float bc1 = bias.bc1[0], bc2 = bias.bc2[0];
-#pragma unroll
-    for (int j = 1; j < kAmpMaxInFlight; j++) {
-        if (pick == j) {
-            bc1 = bias.bc1[j];
-            bc2 = bias.bc2[j];
-        }
-    }
-    prm.bc1 = bc1;
-    prm.bc2 = bc2;
-
+    amp_pick_bias(prm, bias, (int)head.w);
     bool bad = false;
     if (whole) {
         bad = amp_fused_finish<VEC, NT>(loaded, out, s.first, prm, inv_scale);

@@ -138,6 +138,11 @@ __global__ void __launch_bounds__(BLOCK)
 multi_tensor_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm)
 {
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    // An idle slice leaves here.  (The weight pointer is never null; testing it together with the
+    // count makes the compiler fetch the whole descriptor with one wait, instead of the count
+    // first and, behind the branch and a second wait, the addresses.)
+    const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
+    if ((first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr)) return;
     update_slice<Rule, VEC, NT, false, BLOCK>(ch, slice_shift, prm, 1.0f);
 }
 
@@ -147,6 +152,8 @@ __global__ void __launch_bounds__(BLOCK)
 multi_tensor_sgd_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm)
 {
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
+    if ((first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr)) return;     // as above
     if (prm.momentum > 0.0f && ch.p[kSlotState0] != nullptr)
         update_slice<SgdMomentumRule, VEC, NT, false, BLOCK>(ch, slice_shift, prm, 1.0f);
     else
