@@ -62,7 +62,7 @@ struct AmpBiasTable {
 
 // Phase A: OR over every fp16 gradient element of "exponent field all ones"
 // (+-inf or NaN).  Per lane OR -> wavefront ballot -> one LDS word per wave ->
-// one atomic per workgroup that saw a hit.
+// one store of the step's stamp per workgroup that saw a hit.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
 amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state, int reverse,
@@ -122,13 +122,13 @@ __device__ inline void amp_pick_bias(StepParams &prm, const AmpBiasTable &bias, 
 }
 
 // Phase B: the Adam update on unscaled gradients, skipped as a whole when the
-// flag is set.
+// check stored this step's stamp.
 template <int VEC, bool NT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
                        const AmpDeviceState *__restrict__ state, AmpBiasTable bias, unsigned int stamp)
 {
-    // The state's head (current set, reciprocal of the scale, flag, applied steps) comes with one 16-byte scalar load
+    // The state's head (current set, reciprocal of the scale, overflow stamp, applied steps) comes with one 16-byte scalar load
     // and the chunk descriptor with another, both issued before anything is decided; the bias
     // table sits in the kernel arguments and its entry comes with an indexed scalar load.
     const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
@@ -197,9 +197,9 @@ __device__ inline bool amp_fused_finish(const FusedLoaded<N> &x, const Chunk &ou
 }
 
 // The ping-pong step: one pass.  Reads weights and moments of the current set and the fp16
-// gradients, writes the other set and the fp16 weight copy, and raises the flag when a gradient
-// of its own is +-inf or NaN.  It never looks at the flag: what it writes becomes current only if
-// the epilogue finds the flag clear.
+// gradients, writes the other set and the fp16 weight copy, and stores the step's stamp when a
+// gradient of its own is +-inf or NaN.  Its arithmetic never looks at the stamp: what it writes
+// becomes current only if the epilogue finds that no workgroup stored it.
 // (The state pointer is the first argument and the early exit tests the head: both make the
 // compiler fetch the state's head together with the two descriptors, straight after the kernel
 // arguments, instead of behind the first branch; that shortens the chain of dependent scalar
