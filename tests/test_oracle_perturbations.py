@@ -1,0 +1,92 @@
+"""Each pin in test_oracle_properties.py is shown to bite: oracle.c is rebuilt with ONE plausible mistake (a term
+dropped, epsilon on the other side of the root, the decay folded in at the wrong place, a schedule taken at the wrong
+step, two coefficients swapped, a bound removed) and the pin that is meant to catch it must then fail.  Unperturbed,
+the same pins pass (they are part of this suite).  The perturbed builds live in a temporary folder; the pins run in a
+child process that loads them through GM_ORACLE_SO."""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+PINS = os.path.join(ROOT, "tests", "test_oracle_properties.py")
+
+# (name, text in oracle.c, what it becomes, -k expression of the pins that must fail)
+CASES = [
+    ("NAdam momentum schedule taken at t instead of t + 1",
+     "float exponent = (float)(step + 1) * 0.004f;", "float exponent = (float)(step) * 0.004f;",
+     "test_nadam_momentum_schedule_is_taken_at_t_plus_one"),
+    ("NAdam epsilon inside the root",
+     "        float root = sqrtf(v_hat);              /* :2170 */\n        float den = root + eps;                 /* :2171 */",
+     "        float root = sqrtf(v_hat + eps);\n        float den = root;",
+     "test_nadam_first_step_closed_form_bit_exact or test_epsilon_placement"),
+    ("NAdam gradient term dropped from the look-ahead",
+     "float m_bar = m_term + g_term;          /* :2164 */", "float m_bar = m_term; (void)g_term;",
+     "test_nadam_first_step_closed_form_bit_exact"),
+    ("NAdam decay folded into the gradient",
+     "        float gi = g[i];\n        float m_scaled = m[i] * beta1;          /* :2114 */",
+     "        float gi = g[i] + (weight_decay > 0.0f ? w[i] * weight_decay : 0.0f);\n        float m_scaled = m[i] * beta1;",
+     "test_nadam_first_step_closed_form_bit_exact or test_decay_order"),
+    ("Adam epsilon inside the root",
+     "    float root = sqrtf(v_hat);                 /* :519 */\n    float den = root + eps;                    /* :521 */",
+     "    float root = sqrtf(v_hat + eps);\n    float den = root;",
+     "test_epsilon_placement"),
+    ("RMSProp epsilon outside the root",
+     "            float s_eps = si + eps;\n            den = sqrtf(s_eps);", "            den = sqrtf(si) + eps;",
+     "test_epsilon_placement or test_rmsprop_epsilon_inside"),
+    ("AdaDelta numerator fed by the updated average",
+     "        float a_eps = ai + eps;                /* :1807 */",
+     "        ai = ai * rho + (gi * gi) * omr; float a_eps = ai + eps;",
+     "test_adadelta_second_step"),
+    ("AdaDelta rho and 1 - rho swapped in the update average",
+     "        float d_sq_scaled = d_sq * omr;        /* :1838 */", "        float d_sq_scaled = d_sq * rho;",
+     "test_adadelta_second_step"),
+    ("RMSProp decay folded into the gradient",
+     "        float gi = g[i];\n        float g_sq = gi * gi;                  /* :782 */",
+     "        float gi = g[i] + (weight_decay > 0.0f ? w[i] * weight_decay : 0.0f);\n        float g_sq = gi * gi;",
+     "test_decay_order"),
+    ("AdaGrad decay dropped from the gradient",
+     "            gi = gi + decay;\n        }\n        float g_sq = gi * gi;                  /* :1492 */",
+     "            (void)decay;\n        }\n        float g_sq = gi * gi;",
+     "test_decay_order"),
+    ("RMSProp alpha and 1 - alpha swapped",
+     "        float s_scaled = s[i] * alpha;         /* :785 */\n        float g_sq_scaled = g_sq * oma;        /* :788 */",
+     "        float s_scaled = s[i] * oma;\n        float g_sq_scaled = g_sq * alpha;",
+     "test_rmsprop_second_step_with_decay_bit_exact"),
+    ("loss-scale growth unbounded",
+     "        if (next <= FLT_MAX) st->scale = next;", "        st->scale = next;",
+     "test_amp_scale_stays_finite"),
+]
+
+
+def run_case(case, folder):
+    name, old, new, pins = case
+    src = open(os.path.join(ORACLE_DIR, "oracle.c")).read()
+    if src.count(old) != 1:
+        return name, "the line to perturb was not found exactly once in oracle.c"
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "oracle.c"), "w") as f:
+        f.write(src.replace(old, new))
+    so = os.path.join(folder, "liboracle.so")
+    build = subprocess.run(["gcc", "-O2", "-std=c11", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-fopenmp", "-w",
+                            "-I", ORACLE_DIR, "-shared", "-o", so, os.path.join(folder, "oracle.c"),
+                            os.path.join(ORACLE_DIR, "oracle_lbfgs.c"), "-lm"], capture_output=True, text=True)
+    if build.returncode != 0:
+        return name, "the perturbed oracle did not build: " + build.stderr[-500:]
+    r = subprocess.run([sys.executable, "-m", "pytest", PINS, "-q", "-x", "-k", pins, "-p", "no:cacheprovider"],
+                       env=dict(os.environ, GM_ORACLE_SO=so), capture_output=True, text=True)
+    if r.returncode == 0:
+        return name, f"NOT caught by: {pins}"
+    if " failed" not in r.stdout:
+        return name, "the pins did not run to a failure: " + (r.stdout + r.stderr)[-500:]
+    return name, None
+
+
+def test_every_perturbation_of_the_oracle_fails_its_pin(tmp_path):
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        results = list(pool.map(lambda ic: run_case(ic[1], str(tmp_path / f"case{ic[0]}")), enumerate(CASES)))
+    problems = [f"{name}: {why}" for name, why in results if why]
+    assert not problems, "\n".join(problems)
