@@ -56,6 +56,43 @@ CASES = [
      "        float s_scaled = s[i] * alpha;         /* :785 */\n        float g_sq_scaled = g_sq * oma;        /* :788 */",
      "        float s_scaled = s[i] * oma;\n        float g_sq_scaled = g_sq * alpha;",
      "test_rmsprop_second_step_with_decay_bit_exact"),
+    ("SGD Nesterov look-ahead built from the old momentum",
+     "                float t1 = momentum * mi;", "                float t1 = momentum * m[i];",
+     "test_sgd_closed_forms"),
+    ("SGD momentum with dampening",
+     "            float mi = scaled + gi;          /* :248 */", "            float mi = scaled + gi * (1.0f - momentum);",
+     "test_sgd_closed_forms"),
+    ("SGD decay applied to the weight instead of the gradient",
+     "            float decay = wi * weight_decay;\n            gi = gi + decay;\n        }\n        if (use_momentum) {",
+     "            wi = wi - lr * wi * weight_decay;\n        }\n        if (use_momentum) {",
+     "test_sgd_closed_forms or test_decay_order"),
+    ("Adam second-moment bias correction dropped",
+     "    float v_hat = vi / bc2;                    /* :514 */", "    float v_hat = vi; (void)bc2;",
+     "test_adam_first_step_closed_form or test_adam_against_float64_formula_and_decay_order"),
+    ("Adam beta1 and 1 - beta1 swapped",
+     "    float m_scaled = *m * beta1;               /* :484 */\n    float g_scaled = g * one_minus_beta1;      /* :487 */",
+     "    float m_scaled = *m * one_minus_beta1;\n    float g_scaled = g * beta1;",
+     "test_adam_first_step_closed_form"),
+    ("Adam decay folded into the gradient",
+     "    float m_scaled = *m * beta1;               /* :484 */",
+     "    if (weight_decay > 0.0f) g = g + wi * weight_decay;\n    float m_scaled = *m * beta1;",
+     "test_adam_against_float64_formula_and_decay_order or test_decay_order"),
+    ("Adam decay scaled by nothing (applied after the learning rate)",
+     "    float scaled = upd * lr;                   /* :543 */\n    *w = wi - scaled;                          /* :548 */",
+     "    float scaled = (upd - (weight_decay > 0.0f ? wi * weight_decay : 0.0f)) * lr;\n    *w = wi - scaled - (weight_decay > 0.0f ? wi * weight_decay : 0.0f);",
+     "test_adam_against_float64_formula_and_decay_order or test_decay_order"),
+    ("AdaGrad epsilon inside the root",
+     "        float root = sqrtf(si);                /* :1501 */\n        float den = root + eps;                /* :1503 */",
+     "        float root = sqrtf(si + eps);\n        float den = root;",
+     "test_adagrad_closed_form_and_monotone_state or test_epsilon_placement"),
+    ("AdaGrad product formed before the quotient",
+     "        float alr = lr / den;                  /* :1506 */\n        float upd = alr * gi;                  /* :1512 */",
+     "        float alr = lr * gi;\n        float upd = alr / den;",
+     "test_adagrad_closed_form_and_monotone_state"),
+    ("AdaDelta epsilon outside the roots",
+     "        float s_eps = si + eps;                /* :1800 */\n        float rms_g = sqrtf(s_eps);            /* :1803 */",
+     "        float s_eps = si;\n        float rms_g = sqrtf(s_eps) + eps;",
+     "test_adadelta_first_step_closed_form"),
     ("loss-scale growth unbounded",
      "        if (next <= FLT_MAX) st->scale = next;", "        st->scale = next;",
      "test_amp_scale_stays_finite"),
