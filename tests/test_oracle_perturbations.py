@@ -93,27 +93,44 @@ CASES = [
      "        float s_eps = si + eps;                /* :1800 */\n        float rms_g = sqrtf(s_eps);            /* :1803 */",
      "        float s_eps = si;\n        float rms_g = sqrtf(s_eps) + eps;",
      "test_adadelta_first_step_closed_form"),
+    ("mixed precision: clean-step counter not reset by a dropped step",
+     "        st->growth_tracker = 0;\n        return 1;", "        return 1;",
+     "test_amp_skip_and_scale_sequence_against_brute_force"),
+    ("mixed precision: a dropped step advances the step count",
+     "        st->growth_tracker = 0;\n        return 1;", "        st->growth_tracker = 0;\n        st->step_count += 1;\n        return 1;",
+     "test_amp_skip_and_scale_sequence_against_brute_force"),
+    ("mixed precision: growth one step late",
+     "    if (st->growth_tracker == st->growth_interval) {", "    if (st->growth_tracker > st->growth_interval) {",
+     "test_amp_skip_and_scale_sequence_against_brute_force"),
+    ("mixed precision: NaN gradients not treated as overflow",
+     "            local |= ((g[i] & 0x7C00u) == 0x7C00u);", "            local |= ((g[i] & 0x7FFFu) == 0x7C00u);",
+     "test_amp_skip_and_scale_sequence_against_brute_force"),
+    ("mixed precision: no backoff on a dropped step",
+     "        if (next >= FLT_MIN) st->scale = next;        /* the scale stays a normal number */", "        (void)next;",
+     "test_amp_skip_and_scale_sequence_against_brute_force"),
     ("loss-scale growth unbounded",
      "        if (next <= FLT_MAX) st->scale = next;", "        st->scale = next;",
      "test_amp_scale_stays_finite"),
 ]
 
 
-def run_case(case, folder):
+def run_case(case, folder, source="oracle.c", pin_file=PINS):
     name, old, new, pins = case
-    src = open(os.path.join(ORACLE_DIR, "oracle.c")).read()
+    src = open(os.path.join(ORACLE_DIR, source)).read()
     if src.count(old) != 1:
-        return name, "the line to perturb was not found exactly once in oracle.c"
+        return name, f"the line to perturb was not found exactly once in {source}"
     os.makedirs(folder, exist_ok=True)
-    with open(os.path.join(folder, "oracle.c"), "w") as f:
+    files = {f: os.path.join(ORACLE_DIR, f) for f in ("oracle.c", "oracle_lbfgs.c")}
+    files[source] = os.path.join(folder, source)
+    with open(files[source], "w") as f:
         f.write(src.replace(old, new))
     so = os.path.join(folder, "liboracle.so")
     build = subprocess.run(["gcc", "-O2", "-std=c11", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-fopenmp", "-w",
-                            "-I", ORACLE_DIR, "-shared", "-o", so, os.path.join(folder, "oracle.c"),
-                            os.path.join(ORACLE_DIR, "oracle_lbfgs.c"), "-lm"], capture_output=True, text=True)
+                            "-I", ORACLE_DIR, "-shared", "-o", so, files["oracle.c"], files["oracle_lbfgs.c"], "-lm"],
+                           capture_output=True, text=True)
     if build.returncode != 0:
         return name, "the perturbed oracle did not build: " + build.stderr[-500:]
-    r = subprocess.run([sys.executable, "-m", "pytest", PINS, "-q", "-x", "-k", pins, "-p", "no:cacheprovider"],
+    r = subprocess.run([sys.executable, "-m", "pytest", pin_file, "-q", "-x", "-k", pins, "-p", "no:cacheprovider"],
                        env=dict(os.environ, GM_ORACLE_SO=so), capture_output=True, text=True)
     if r.returncode == 0:
         return name, f"NOT caught by: {pins}"
@@ -125,5 +142,30 @@ def run_case(case, folder):
 def test_every_perturbation_of_the_oracle_fails_its_pin(tmp_path):
     with ThreadPoolExecutor(max_workers=4) as pool:
         results = list(pool.map(lambda ic: run_case(ic[1], str(tmp_path / f"case{ic[0]}")), enumerate(CASES)))
+    problems = [f"{name}: {why}" for name, why in results if why]
+    assert not problems, "\n".join(problems)
+
+
+LBFGS_PINS = os.path.join(ROOT, "tests", "test_oracle_lbfgs.py")
+LBFGS_CASES = [
+    ("recursion started from +g", "dir[i][k] = -g[i][k];", "dir[i][k] = g[i][k];", "test"),
+    ("first loop adds alpha y", "dir[i][k] = dir[i][k] - alpha_j * yj[i][k];", "dir[i][k] = dir[i][k] + alpha_j * yj[i][k];", "test"),
+    ("second loop uses alpha + beta", "const float coeff = alpha[j] - beta;", "const float coeff = alpha[j] + beta;", "test"),
+    ("direction not negated after the recursion", "dir[i][k] = -dir[i][k];", "dir[i][k] = dir[i][k];", "test"),
+    ("old gradient kept until after y is formed", "        memcpy(old_g[i], g[i], n[i] * sizeof(float));\n    }",
+     "    }", "test"),
+    ("history walked newest-last in the first loop",
+     "    for (int j = history_count - 1; j >= 0; j--) {\n        const int idx = (history_index - history_count + j + history_size) % history_size;",
+     "    for (int j = history_count - 1; j >= 0; j--) {\n        const int idx = (history_index - 1 - j + history_size) % history_size;",
+     "test"),
+    ("current step stored into the previous slot", "    const int cur = history_index;",
+     "    const int cur = (history_index - 1 + history_size) % history_size;", "test"),
+]
+
+
+def test_every_perturbation_of_the_lbfgs_oracle_fails_its_pins(tmp_path):
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        results = list(pool.map(lambda ic: run_case(ic[1], str(tmp_path / f"case{ic[0]}"), "oracle_lbfgs.c", LBFGS_PINS),
+                                enumerate(LBFGS_CASES)))
     problems = [f"{name}: {why}" for name, why in results if why]
     assert not problems, "\n".join(problems)
