@@ -32,6 +32,13 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+STATE_PHASES = (512 << 10, 1536 << 10, 1 << 20)     # host/memory_manager.hpp, kStatePhases
+
+
+def state_phase(j, nbytes):
+    """Where MemoryManager.AllocateStateBuffer starts the j-th state buffer of a tensor: at its own phase modulo
+    2 MiB when the request falls into the 16 MiB tier or above (more than 4 MiB), anywhere otherwise."""
+    return STATE_PHASES[j % len(STATE_PHASES)] if nbytes > (4 << 20) else None
 
 # algorithmic bytes per parameter per step: every stream read once and / or written once
 BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelta": 28, "nadam": 28,
@@ -291,6 +298,61 @@ def bench_lbfgs(args, pkg, dev):
     print(json.dumps(result))
 
 
+def bench_placement(args, pkg, dev):
+    """Where the state buffers start against where hipMalloc would put them: the fp32 Adam step over the 1.012B list
+    in several layouts of device memory (a spacer of a different size in front of the lists each time, which moves
+    every later allocation), once with the two moment streams allocated plainly, exact sizes, stream after stream,
+    and once with them at the phases the optimizers use.  Same weights and gradients for both."""
+    lib, D = dev.lib, dev.handle
+    from workloads import transformer_block_sizes
+    sizes = transformer_block_sizes()
+    n, params = len(sizes), sum(sizes)
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)
+    bs = pkg.int_array([4 * s for s in sizes])
+    rows = []
+    spacers = [0, 3 << 20, 34 << 20, 129 << 20, (512 << 20) + (6 << 20), (1 << 30) + (77 << 20)]
+    for spacer in spacers:
+        pad = dev.alloc(spacer) if spacer else 0
+        w = [dev.alloc(4 * s) for s in sizes]
+        g = [dev.alloc(4 * s) for s in sizes]
+        plain = [[dev.alloc(4 * s, zero=True) for s in sizes] for _ in range(2)]
+        placed = [[dev.alloc(4 * s, zero=True, phase=state_phase(j, 4 * s)) for s in sizes] for j in range(2)]
+        for k, s in enumerate(sizes):
+            lib.gm_fill_normal_f32(D, w[k], s, 0x6D657461 + k, 0.0, 0.02)
+            lib.gm_fill_normal_f32(D, g[k], s, 0x12345 + k, 0.0, 1e-4)
+        dev.synchronize()
+        cw, cg = pkg.handle_array(w), pkg.handle_array(g)
+        row = {"spacer_bytes": spacer}
+        t = {"t": 0}
+        for name, states in (("plain", plain), ("placed", placed), ("plain_again", plain), ("placed_again", placed)):
+            cm, cv = pkg.handle_array(states[0]), pkg.handle_array(states[1])
+
+            def launch():
+                t["t"] += 1
+                rc = lib.execute_adam_step_mpsgraph(D, cw, cg, cm, cv, n, bs, hyper["lr"], hyper["beta1"], hyper["beta2"],
+                                                    hyper["eps"], hyper["weight_decay"], t["t"])
+                if rc != 0:
+                    raise RuntimeError(f"adam step failed rc={rc}: {lib.gm_last_error().decode()}")
+            _, ms = time_steps(dev, launch, args.steps, max(args.warmup, 5))
+            row[name] = {"kernel_ms": ms, "frac": params * 28 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        rows.append(row)
+        for h in w + g + plain[0] + plain[1] + placed[0] + placed[1] + ([pad] if pad else []):
+            dev.free(h)
+    mean = lambda key: sum((r[key]["frac"] + r[key + "_again"]["frac"]) / 2 for r in rows) / len(rows)
+    result = {"metric": "fraction of HBM peak of the fp32 Adam step by placement of the state buffers",
+              "unit": "fraction of 8 TB/s", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 5),
+              "config": {"workload": "placement: 1,012,301,824 params in 400 tensors, six layouts of device memory",
+                         "state_phases": list(STATE_PHASES[:2])},
+              "plain_mean": mean("plain"), "placed_mean": mean("placed"),
+              "plain_range": [min(min(r["plain"]["frac"], r["plain_again"]["frac"]) for r in rows),
+                              max(max(r["plain"]["frac"], r["plain_again"]["frac"]) for r in rows)],
+              "placed_range": [min(min(r["placed"]["frac"], r["placed_again"]["frac"]) for r in rows),
+                               max(max(r["placed"]["frac"], r["placed_again"]["frac"]) for r in rows)],
+              "layouts": rows}
+    dev.close()
+    print(json.dumps(result))
+
+
 def bench_primitives(args, pkg, dev):
     """Buffer primitives of the boundary on one large buffer each: zero fill, fp32 <-> fp16 conversion,
     device-to-device copy (HBM-bound, timed with HIP events on the library's stream) and the host copies
@@ -445,7 +507,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="", choices=[""] + sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives", "all"],
+    ap.add_argument("--workload", default="", choices=[""] + sorted(WORKLOADS) + sorted(LBFGS_WORKLOADS) + ["primitives", "placement", "all"],
                     help="one workload in this process.  Default: the five benchmark configurations in turn, each in a "
                          "process of its own; the line printed is the headline configuration's (c5) with the others "
                          "under 'configs'.  'all': the same plus the L-BFGS workloads and the buffer primitives")
@@ -488,6 +550,8 @@ def main():
         return bench_lbfgs(args, pkg, dev)
     if args.workload == "primitives":
         return bench_primitives(args, pkg, dev)
+    if args.workload == "placement":
+        return bench_placement(args, pkg, dev)
 
     desc, sizes_fn, rule, hyper, grad_std = WORKLOADS[args.workload]
     if args.rule and args.rule != rule:
@@ -502,7 +566,9 @@ def main():
     # ---- synthetic data, generated on the device ----
     w = [dev.alloc(4 * s) for s in sizes]
     g = [dev.alloc(4 * s) for s in sizes]
-    states = [[dev.alloc(4 * s, zero=True) for s in sizes] for _ in range(nstate)]
+    # state buffers as the optimizers allocate them (memory.MemoryManager.AllocateStateBuffer): the j-th state of a
+    # tensor starts at its own phase modulo 2 MiB, away from the weights' and gradients' 2 MiB-aligned starts
+    states = [[dev.alloc(4 * s, zero=True, phase=state_phase(j, 4 * s)) for s in sizes] for j in range(nstate)]
     for k, s in enumerate(sizes):
         lib.gm_fill_normal_f32(D, w[k], s, 0x6D657461 + k, 0.0, 0.02)
         lib.gm_fill_normal_f32(D, g[k], s, 0x12345 + k, 0.0, grad_std)
@@ -568,6 +634,8 @@ def main():
                      "copy_kernel_gbs": copy_gbs,
                      "frac_of_copy_kernel": achieved / copy_gbs},
     }
+    result["config"]["state_placement"] = ("state buffers of more than 4 MiB start at phases of their own modulo 2 MiB, "
+                                            "as the optimizers allocate them: " + ", ".join(str(p) for p in STATE_PHASES[:nstate]))
     footprint = params * 4 * (2 + nstate)            # every stream of the step, in bytes
     if footprint < 256 * 1024 * 1024:
         result["roofline"]["note"] = (f"the step's {footprint / 1e6:.0f} MB stay in the 256 MB memory-side cache between "
@@ -630,7 +698,9 @@ def main():
         lib.gm_amp_state_destroy(amp)
 
         # ---- the same step in one pass over ping-pong state (two sets of weights and moments) ----
-        shadow = [[dev.alloc(4 * s) for s in sizes] for _ in range(3)]
+        # the second set as EnablePingPong allocates it: weights 1 MiB off, moments at their counterparts' phases
+        shadow = [[dev.alloc(4 * s, phase=ph if 4 * s > (4 << 20) else None) for s in sizes]
+                  for ph in (1 << 20, STATE_PHASES[0], STATE_PHASES[1])]
         c_shadow = [pkg.handle_array(hs) for hs in shadow]
         amp2 = lib.gm_amp_state_create(D, 65536.0, 2.0, 0.5, 2000)
         lib.gm_amp_state_set_step_count(amp2, amp_t["t"])

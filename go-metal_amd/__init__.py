@@ -69,6 +69,7 @@ ABI = {
     "gm_amp_state_max_in_flight": (i, [u]),
     "execute_adam_amp_step_async": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, u]),
     "execute_adam_amp_step": (i, [u, up, up, up, up, up, i, ip, f, f, f, f, f, i, u, ip, fp, ip]),
+    "gm_allocate_buffer_phased": (u, [u, i, i, i]),
     "execute_adam_step_noalloc": (i, [u, up, up, up, up, i, ip, f, f, f, f, f, i]),
     "gm_plan_cache_stats": (i, [u, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ip]),
     "execute_adam_amp_step_fused": (i, [u, up, up, up, up, up, up, up, up, i, ip, f, f, f, f, f, i, u, ip, fp, ip, ip]),
@@ -221,8 +222,12 @@ class Device:
         self._owned = []
 
     # ---- buffers ----
-    def alloc(self, nbytes, zero=False):
-        h = self.lib.allocate_metal_buffer(self.handle, int(nbytes), 1)
+    def alloc(self, nbytes, zero=False, phase=None):
+        """phase: start the buffer at this many bytes modulo 2 MiB (gm_allocate_buffer_phased)."""
+        if phase is None:
+            h = self.lib.allocate_metal_buffer(self.handle, int(nbytes), 1)
+        else:
+            h = self.lib.gm_allocate_buffer_phased(self.handle, int(nbytes), 1, int(phase))
         if not h:
             raise MemoryError(f"allocate_metal_buffer({nbytes}) failed: " +
                               self.lib.gm_last_error().decode())

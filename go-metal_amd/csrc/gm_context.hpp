@@ -79,8 +79,10 @@ Context *resolve_device(uintptr_t device);
 bool make_current(Context *ctx);
 
 // ---- buffer registry: handle (device address) -> allocation length ----
-void registry_add(uintptr_t buffer, size_t bytes);
-void registry_remove(uintptr_t buffer);
+// base: the address to hand back to hipFree when it differs from the handle (0: the handle itself)
+void registry_add(uintptr_t buffer, size_t bytes, uintptr_t base = 0);
+// Forgets the handle and returns the address to free (0 when the handle is unknown).
+uintptr_t registry_remove(uintptr_t buffer);
 // 0 when the handle is not one of ours.
 size_t registry_length(uintptr_t buffer);
 

@@ -84,26 +84,34 @@ Context *resolve_device(uintptr_t device)
 bool make_current(Context *ctx) { return hip_ok(hipSetDevice(ctx->device_id), "hipSetDevice"); }
 
 // -------------------------------------------------------------- registry ----
+struct Allocation {
+    size_t bytes;        // usable length from the handle on
+    uintptr_t base;      // what hipMalloc returned (the handle itself unless the buffer is phased)
+};
 static std::mutex g_reg_mu;
-static std::unordered_map<uintptr_t, size_t> g_reg;
+static std::unordered_map<uintptr_t, Allocation> g_reg;
 
-void registry_add(uintptr_t buffer, size_t bytes)
+void registry_add(uintptr_t buffer, size_t bytes, uintptr_t base)
 {
     std::lock_guard<std::mutex> lk(g_reg_mu);
-    g_reg[buffer] = bytes;
+    g_reg[buffer] = Allocation{bytes, base ? base : buffer};
 }
 
-void registry_remove(uintptr_t buffer)
+uintptr_t registry_remove(uintptr_t buffer)
 {
     std::lock_guard<std::mutex> lk(g_reg_mu);
-    g_reg.erase(buffer);
+    auto it = g_reg.find(buffer);
+    if (it == g_reg.end()) return 0;
+    const uintptr_t base = it->second.base;
+    g_reg.erase(it);
+    return base;
 }
 
 size_t registry_length(uintptr_t buffer)
 {
     std::lock_guard<std::mutex> lk(g_reg_mu);
     auto it = g_reg.find(buffer);
-    return it == g_reg.end() ? 0 : it->second;
+    return it == g_reg.end() ? 0 : it->second.bytes;
 }
 
 // --------------------------------------------------------------- kernels ----
@@ -448,10 +456,43 @@ try {
         plans_forget_range(ctx, buffer, len);
         lbfgs_forget_range(buffer, len);
     }
-    registry_remove(buffer);
-    (void)hipFree(reinterpret_cast<void *>(buffer));   // hipFree waits for work in flight
+    const uintptr_t base = registry_remove(buffer);
+    if (base) (void)hipFree(reinterpret_cast<void *>(base));   // hipFree waits for work in flight
 } catch (...) {
     note_exception();
+}
+
+// Where a buffer starts decides which HBM channels and banks its elements fall into.  Buffers from
+// hipMalloc share their low address bits (large ones are 2 MiB aligned), so element i of a
+// tensor's weight, gradient and state buffers all land on the same channel at the same moment
+// and a workgroup's four loads queue up behind each other.  Measured on MI355X, Adam over the
+// 1.012B-parameter list: 82.0 % of peak with every stream at the same phase, 83.1 % with the two
+// state streams 512 KiB and 1.5 MiB off (mod 2 MiB); 78.9 % to 84.4 % over flat arrays depending
+// on the spacing alone (address bits 12, 19 and 20 separate streams, bits 13 and 21 set them
+// against each other).  The optimizers own their state buffers and ask for them here.
+constexpr size_t kPhasePeriod = 2u << 20;
+constexpr size_t kPhasedMinBytes = 1u << 20;      // below this the phase is ignored: nothing to gain, 2 MiB to lose
+
+uintptr_t gm_allocate_buffer_phased(uintptr_t device, int size, int device_type, int phase_bytes)
+try {
+    if (phase_bytes < 0 || (size_t)phase_bytes >= kPhasePeriod || phase_bytes % 256 != 0) {
+        set_error("a phase is a multiple of 256 bytes below %zu (got %d)", kPhasePeriod, phase_bytes);
+        return 0;
+    }
+    if (device == 0 || size <= 0) return 0;
+    if ((size_t)size < kPhasedMinBytes) return allocate_metal_buffer(device, size, device_type);
+    Context *ctx = resolve_device(device);
+    if (!ctx || !make_current(ctx)) return 0;
+    const size_t aligned = ((size_t)size + 15) / 16 * 16;
+    void *p = nullptr;
+    if (!hip_ok(hipMalloc(&p, aligned + kPhasePeriod), "hipMalloc")) return 0;
+    const uintptr_t base = reinterpret_cast<uintptr_t>(p);
+    const uintptr_t handle = base + (((uintptr_t)phase_bytes + kPhasePeriod - base % kPhasePeriod) % kPhasePeriod);
+    registry_add(handle, aligned, base);
+    return handle;
+} catch (...) {
+    note_exception();
+    return 0;
 }
 
 size_t gm_buffer_length(uintptr_t buffer) { return registry_length(buffer); }

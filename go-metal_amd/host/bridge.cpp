@@ -65,6 +65,13 @@ std::pair<Pointer, Error> AllocateMetalBuffer(Pointer device, int size, DeviceTy
     return {P(buffer), ""};
 }
 
+std::pair<Pointer, Error> AllocateMetalBufferPhased(Pointer device, int size, DeviceType deviceType, int phase)
+{
+    uintptr_t buffer = gm_allocate_buffer_phased(H(device), size, (int)deviceType, phase);
+    if (buffer == 0) return {nullptr, Errorf("failed to allocate Metal buffer of size %d", size)};
+    return {P(buffer), ""};
+}
+
 void DeallocateMetalBuffer(Pointer buffer)
 {
     if (buffer != nullptr) deallocate_metal_buffer(H(buffer));

@@ -27,6 +27,8 @@ void DestroyMetalDevice(Pointer device);                                        
 std::pair<Pointer, Error> CreateCommandQueue(Pointer device);                       // bridge.go:1676
 void ReleaseCommandQueue(Pointer queue);                                            // bridge.go:1690
 std::pair<Pointer, Error> AllocateMetalBuffer(Pointer device, int size, DeviceType deviceType);  // bridge.go:729
+// allocate_metal_buffer with the buffer's start placed at `phase` bytes modulo 2 MiB (no counterpart in the reference)
+std::pair<Pointer, Error> AllocateMetalBufferPhased(Pointer device, int size, DeviceType deviceType, int phase);
 void DeallocateMetalBuffer(Pointer buffer);                                         // bridge.go:744
 Error ZeroMetalBuffer(Pointer device, Pointer buffer, int size);                    // bridge.go:1039
 Error CopyFloat32ArrayToMetalBuffer(Pointer buffer, const std::vector<float> &data);  // bridge.go:1069

@@ -134,11 +134,20 @@ void gmo_set_pool_byte_budget(size_t bytes) { memory::SetPoolByteBudget(bytes); 
 int gmo_pool_stats(uintptr_t mm, int pool_size, int *available, int *allocated, int *max_size)
 try {
     if (!mm) return -1;
+    // buffers of one size are pooled apart by the phase they start at: the figures are summed over those pools
     auto stats = MM(mm)->Stats();
-    auto it = stats.find(memory::PoolKey{pool_size, memory::GPU});
-    if (it == stats.end()) return -1;
     int a = 0, b = 0, c = 0;
-    if (std::sscanf(it->second.c_str(), "available=%d, allocated=%d, max=%d", &a, &b, &c) != 3) return -1;
+    bool found = false;
+    for (const auto &kv : stats) {
+        if (kv.first.Size != pool_size || kv.first.Device != memory::GPU) continue;
+        int pa = 0, pb = 0, pc = 0;
+        if (std::sscanf(kv.second.c_str(), "available=%d, allocated=%d, max=%d", &pa, &pb, &pc) != 3) return -1;
+        a += pa;
+        b += pb;
+        c = pc > c ? pc : c;
+        found = true;
+    }
+    if (!found) return -1;
     if (available) *available = a;
     if (allocated) *allocated = b;
     if (max_size) *max_size = c;

@@ -32,7 +32,7 @@ int calculateMaxPoolSize(int bufferSize)
     return (int)capped > ref ? (int)capped : ref;
 }
 
-static std::pair<Pointer, Error> allocateMetalBuffer(int size, DeviceType device)
+static std::pair<Pointer, Error> allocateMetalBuffer(int size, DeviceType device, int phase)
 {
     // manager.go:263-281: the device comes from the global manager
     MemoryManager *global = GetGlobalMemoryManager();
@@ -44,13 +44,14 @@ static std::pair<Pointer, Error> allocateMetalBuffer(int size, DeviceType device
     case PersistentGPU: cgoDev = cgo_bridge::PersistentGPU; break;
     default: cgoDev = cgo_bridge::GPU; break;
     }
+    if (phase != 0) return cgo_bridge::AllocateMetalBufferPhased(global->device(), size, cgoDev, phase);
     return cgo_bridge::AllocateMetalBuffer(global->device(), size, cgoDev);
 }
 
 static void deallocateMetalBuffer(Pointer buffer) { cgo_bridge::DeallocateMetalBuffer(buffer); }
 
-BufferPool::BufferPool(int bufferSize, int maxSize, DeviceType device)
-    : maxSize_(maxSize), bufferSize_(bufferSize), device_(device)
+BufferPool::BufferPool(int bufferSize, int maxSize, DeviceType device, int phase)
+    : maxSize_(maxSize), bufferSize_(bufferSize), device_(device), phase_(phase)
 {
 }
 
@@ -71,7 +72,7 @@ std::pair<Pointer, Error> BufferPool::Get()
         if (allocated_ >= maxSize_) return {nullptr, Errorf("buffer pool at capacity (%d)", maxSize_)};
         allocated_++;
     }
-    auto [buffer, err] = allocateMetalBuffer(bufferSize_, device_);
+    auto [buffer, err] = allocateMetalBuffer(bufferSize_, device_, phase_);
     if (!err.empty()) {
         std::lock_guard<std::mutex> lk(mutex_);
         allocated_--;
@@ -121,27 +122,31 @@ BufferPool *MemoryManager::getOrCreatePool(const PoolKey &key)
     std::lock_guard<std::mutex> lk(poolsMutex_);
     auto it = pools_.find(key);
     if (it != pools_.end()) return it->second.get();
-    auto pool = std::make_unique<BufferPool>(key.Size, calculateMaxPoolSize(key.Size), key.Device);
+    auto pool = std::make_unique<BufferPool>(key.Size, calculateMaxPoolSize(key.Size), key.Device, key.Phase);
     BufferPool *raw = pool.get();
     pools_[key] = std::move(pool);
     return raw;
 }
 
-std::pair<Pointer, Error> MemoryManager::GetBuffer(int size, DeviceType device)
+std::pair<Pointer, Error> MemoryManager::GetBuffer(int size, DeviceType device, int phase)
 {
     const int poolSize = findPoolSize(size);
-    BufferPool *pool = getOrCreatePool(PoolKey{poolSize, device});
+    if (poolSize < kPhasedMinBytes) phase = 0;
+    BufferPool *pool = getOrCreatePool(PoolKey{poolSize, device, phase});
     auto [buffer, err] = pool->Get();
     if (!err.empty()) return {nullptr, err};
     std::lock_guard<std::mutex> lk(bufferSizesMutex_);
     bufferSizes_[buffer] = poolSize;
+    if (phase != 0) bufferPhases_[buffer] = phase;
     return {buffer, ""};
 }
 
-void MemoryManager::ReturnBuffer(Pointer buffer, int size, DeviceType device)
+void MemoryManager::ReturnBuffer(Pointer buffer, int size, DeviceType device, int phase)
 {
     if (buffer == nullptr) return;
-    const PoolKey key{findPoolSize(size), device};
+    const int poolSize = findPoolSize(size);
+    if (poolSize < kPhasedMinBytes) phase = 0;
+    const PoolKey key{poolSize, device, phase};
     BufferPool *pool = nullptr;
     {
         std::lock_guard<std::mutex> lk(poolsMutex_);
@@ -152,6 +157,7 @@ void MemoryManager::ReturnBuffer(Pointer buffer, int size, DeviceType device)
     else deallocateMetalBuffer(buffer);   // no pool exists, just deallocate
     std::lock_guard<std::mutex> lk(bufferSizesMutex_);
     bufferSizes_.erase(buffer);
+    bufferPhases_.erase(buffer);
 }
 
 Pointer MemoryManager::AllocateBuffer(int size)
@@ -161,10 +167,25 @@ Pointer MemoryManager::AllocateBuffer(int size)
     return buffer;
 }
 
+Pointer MemoryManager::AllocateStateBuffer(int size, int stateIndex)
+{
+    const int phase = stateIndex >= 0 && stateIndex < 3 ? kStatePhases[stateIndex] : 0;
+    auto [buffer, err] = GetBuffer(size, GPU, phase);
+    if (!err.empty()) return nullptr;
+    return buffer;
+}
+
+Pointer MemoryManager::AllocateBufferAtPhase(int size, int phase)
+{
+    auto [buffer, err] = GetBuffer(size, GPU, phase);
+    if (!err.empty()) return nullptr;
+    return buffer;
+}
+
 void MemoryManager::ReleaseBuffer(Pointer buffer)
 {
     if (buffer == nullptr) return;
-    int size = 0;
+    int size = 0, phase = 0;
     bool exists = false;
     {
         std::lock_guard<std::mutex> lk(bufferSizesMutex_);
@@ -173,12 +194,14 @@ void MemoryManager::ReleaseBuffer(Pointer buffer)
             size = it->second;
             exists = true;
         }
+        auto ph = bufferPhases_.find(buffer);
+        if (ph != bufferPhases_.end()) phase = ph->second;
     }
     if (!exists) {
         size = 4194304;   // 4MB default as fallback (manager.go:309-314)
         std::printf("Warning: releasing untracked buffer %p, using default size %d\n", buffer, size);
     }
-    ReturnBuffer(buffer, size, GPU);
+    ReturnBuffer(buffer, size, GPU, phase);
 }
 
 std::map<PoolKey, std::string> MemoryManager::Stats()

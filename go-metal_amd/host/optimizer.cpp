@@ -251,7 +251,7 @@ std::pair<std::unique_ptr<SGDOptimizerState>, Error> NewSGDOptimizer(const SGDCo
         for (size_t i = 0; i < n; i++) {
             const int size = calculateTensorSize(weightShapes[i]) * 4;
             sgd->bufferSizes[i] = size;
-            Pointer momentumBuffer = memoryManager->AllocateBuffer(size);
+            Pointer momentumBuffer = memoryManager->AllocateStateBuffer(size, 0);
             if (momentumBuffer == nullptr) {
                 releaseAll(memoryManager, sgd->MomentumBuffers);
                 return {nullptr, Errorf("failed to allocate momentum buffer for weight %d", (int)i)};
@@ -356,11 +356,12 @@ static Error allocateMoments(memory::MemoryManager *mm, Pointer device, const Sh
     for (size_t i = 0; i < n; i++) {
         const int size = calculateTensorSize(weightShapes[i]) * 4;
         bufferSizes[i] = size;
-        Pointer momentumBuffer = mm->AllocateBuffer(size);
+        // (the two moments of a tensor start at phases of their own: memory_manager.hpp, kStatePhases)
+        Pointer momentumBuffer = mm->AllocateStateBuffer(size, 0);
         if (momentumBuffer == nullptr)
             return unwind(Errorf("failed to allocate momentum buffer for weight %d", (int)i));
         first[i] = momentumBuffer;
-        Pointer varianceBuffer = mm->AllocateBuffer(size);
+        Pointer varianceBuffer = mm->AllocateStateBuffer(size, 1);
         if (varianceBuffer == nullptr)
             return unwind(Errorf("failed to allocate variance buffer for weight %d", (int)i));
         second[i] = varianceBuffer;
@@ -457,10 +458,12 @@ Error AdamOptimizerState::EnablePingPong()
     for (Pointer w : WeightBuffers)
         if (w == nullptr) return Errorf("weight buffers are not set: call SetWeightBuffers first");
     std::vector<Pointer> *lists[3] = {&ShadowWeightBuffers, &ShadowMomentumBuffers, &ShadowVarianceBuffers};
-    for (auto *list : lists) {
+    const int phases[3] = {memory::kShadowWeightPhase, memory::kStatePhases[0], memory::kStatePhases[1]};
+    for (int k = 0; k < 3; k++) {
+        auto *list = lists[k];
         list->assign(bufferSizes.size(), nullptr);
         for (size_t i = 0; i < bufferSizes.size(); i++) {
-            (*list)[i] = memoryManager->AllocateBuffer(bufferSizes[i]);
+            (*list)[i] = memoryManager->AllocateBufferAtPhase(bufferSizes[i], phases[k]);
             if ((*list)[i] == nullptr) {
                 for (auto *undo : lists) {
                     releaseAll(memoryManager, *undo);
@@ -703,17 +706,17 @@ std::pair<std::unique_ptr<RMSPropOptimizerState>, Error> NewRMSPropOptimizer(con
     for (size_t i = 0; i < n; i++) {
         const int size = calculateTensorSize(weightShapes[i]) * 4;
         r->bufferSizes[i] = size;
-        Pointer s = memoryManager->AllocateBuffer(size);
+        Pointer s = memoryManager->AllocateStateBuffer(size, 0);
         if (s == nullptr)
             return unwind(Errorf("failed to allocate squared gradient average buffer for weight %d", (int)i));
         r->SquaredGradAvgBuffers[i] = s;
         if (config.Momentum > 0.0f) {
-            Pointer b = memoryManager->AllocateBuffer(size);
+            Pointer b = memoryManager->AllocateStateBuffer(size, 1);
             if (b == nullptr) return unwind(Errorf("failed to allocate momentum buffer for weight %d", (int)i));
             r->MomentumBuffers[i] = b;
         }
         if (config.Centered) {
-            Pointer ga = memoryManager->AllocateBuffer(size);
+            Pointer ga = memoryManager->AllocateStateBuffer(size, 2);
             if (ga == nullptr)
                 return unwind(Errorf("failed to allocate gradient average buffer for weight %d", (int)i));
             r->GradientAvgBuffers[i] = ga;
@@ -854,7 +857,7 @@ std::pair<std::unique_ptr<AdaGradOptimizerState>, Error> NewAdaGradOptimizer(con
     a->bufferSizes.assign(n, 0);
     for (size_t i = 0; i < n; i++) {
         a->bufferSizes[i] = calculateTensorSize(weightShapes[i]) * 4;
-        Pointer s = memoryManager->AllocateBuffer(a->bufferSizes[i]);
+        Pointer s = memoryManager->AllocateStateBuffer(a->bufferSizes[i], 0);
         if (s == nullptr) {
             a->Cleanup();
             return {nullptr, Errorf("failed to allocate squared gradient average buffer for weight %d", (int)i)};
@@ -967,13 +970,13 @@ std::pair<std::unique_ptr<AdaDeltaOptimizerState>, Error> NewAdaDeltaOptimizer(c
     a->bufferSizes.assign(n, 0);
     for (size_t i = 0; i < n; i++) {
         a->bufferSizes[i] = calculateTensorSize(weightShapes[i]) * 4;
-        Pointer s = memoryManager->AllocateBuffer(a->bufferSizes[i]);
+        Pointer s = memoryManager->AllocateStateBuffer(a->bufferSizes[i], 0);
         if (s == nullptr) {
             a->Cleanup();
             return {nullptr, Errorf("failed to allocate squared gradient average buffer for weight %d", (int)i)};
         }
         a->squaredGradAvgBuffers[i] = s;
-        Pointer u = memoryManager->AllocateBuffer(a->bufferSizes[i]);
+        Pointer u = memoryManager->AllocateStateBuffer(a->bufferSizes[i], 1);
         if (u == nullptr) {
             a->Cleanup();
             return {nullptr, Errorf("failed to allocate squared update average buffer for weight %d", (int)i)};

@@ -342,6 +342,16 @@ int execute_adam_amp_step_fused_async(uintptr_t device, uintptr_t *weight_a, uin
  * Waits for every step in flight.  -16: nil state; -6: HIP error. */
 int gm_amp_state_current_set(uintptr_t amp_state);
 
+/* allocate_metal_buffer with a say in where the buffer starts: the handle's address is congruent to
+ * phase_bytes modulo 2 MiB (phase_bytes: a multiple of 256 below 2 MiB).  No counterpart in the
+ * reference.  Buffers that start at the same phase put element i of each of them on the same HBM
+ * channel; the optimizers place their state buffers at phases of their own (512 KiB, 1.5 MiB, 1 MiB
+ * for the first, second and third state of a tensor), which is worth a point of bandwidth for
+ * Adam over the 1.012B-parameter list.  Requests under 1 MiB ignore the phase; larger ones cost
+ * 2 MiB more than their size.  The handle is freed with deallocate_metal_buffer and has the
+ * length `size` for every range check.  0 on failure, like allocate_metal_buffer. */
+uintptr_t gm_allocate_buffer_phased(uintptr_t device, int size, int device_type, int phase_bytes);
+
 /* execute_adam_step_mpsgraph for callers that cannot allocate.  No counterpart in the reference:
  * it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc.  Same arguments, arithmetic, update kernel and results as execute_adam_step_mpsgraph;

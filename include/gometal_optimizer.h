@@ -32,7 +32,8 @@ int       gmo_find_pool_size(uintptr_t mm, int size);               /* findPoolS
 int       gmo_calculate_max_pool_size(int buffer_size);             /* manager.go:210, byte-budget extension */
 int       gmo_reference_max_pool_size(int buffer_size);             /* manager.go:210 cap table verbatim */
 void      gmo_set_pool_byte_budget(size_t bytes);
-/* BufferPool.Stats of the pool holding buffers of pool_size; -1 if that pool does not exist. */
+/* BufferPool.Stats of the pools holding buffers of pool_size (buffers placed at a phase are pooled apart: available
+ * and allocated are summed over those pools, max_size is one pool's cap); -1 if no such pool exists. */
 int       gmo_pool_stats(uintptr_t mm, int pool_size, int *available, int *allocated, int *max_size);
 
 /* ---- package optimizer ---- */

@@ -162,11 +162,32 @@ uintptr_t allocate_metal_buffer(uintptr_t device, int size, int)
     return reinterpret_cast<uintptr_t>(p);
 }
 
+// The stand-in keeps exact-length heap blocks (so that overruns land in a red zone) and therefore cannot
+// place a buffer at a phase; it checks the argument as the library does and remembers what was asked for.
+std::map<uintptr_t, int> g_requested_phase;
+uintptr_t gm_allocate_buffer_phased(uintptr_t device, int size, int device_type, int phase_bytes)
+{
+    if (phase_bytes < 0 || phase_bytes >= (2 << 20) || phase_bytes % 256 != 0) return 0;
+    const uintptr_t h = allocate_metal_buffer(device, size, device_type);
+    if (h != 0 && size >= (1 << 20)) {
+        std::lock_guard<std::mutex> lk(g_mu);
+        g_requested_phase[h] = phase_bytes;
+    }
+    return h;
+}
+int cpu_device_requested_phase(uintptr_t buffer)
+{
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_requested_phase.find(buffer);
+    return it == g_requested_phase.end() ? -1 : it->second;
+}
+
 void deallocate_metal_buffer(uintptr_t buffer)
 {
     {
         std::lock_guard<std::mutex> lk(g_mu);
         if (g_buffers.erase(buffer) == 0) return;
+        g_requested_phase.erase(buffer);
     }
     std::free(reinterpret_cast<void *>(buffer));
 }

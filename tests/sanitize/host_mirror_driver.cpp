@@ -175,6 +175,45 @@ static void mixed_precision(uintptr_t device, uintptr_t mm)
     }
 }
 
+extern "C" int cpu_device_requested_phase(uintptr_t buffer);      // cpu_device.cpp
+
+// The state buffers of large tensors are asked for at the phases memory_manager.hpp names (512 KiB, 1.5 MiB,
+// 1 MiB for the first, second and third state), small ones and the callers' own buffers at none, and a
+// released state buffer goes back to the pool of its phase: the next optimizer gets the same handles.
+static void state_buffer_phases(uintptr_t device, uintptr_t mm)
+{
+    const int dims[] = {1100, 1024, 17};            // 1126400 floats = 4.5 MB (the 16 MiB tier), and a small tensor
+    const int ndims[] = {2, 1};
+    float cfg[6] = {0};
+    gmo_default_config(GMO_RMSPROP, cfg);
+    cfg[4] = 0.9f;                                   // momentum
+    cfg[5] = 1.0f;                                   // centered
+    uintptr_t first_handles[3] = {0, 0, 0};
+    const char *kinds[3] = {"squared_grad_avg", "momentum", "gradient_avg"};
+    const int want[3] = {512 << 10, 1536 << 10, 1 << 20};
+    for (int round = 0; round < 2; round++) {
+        uintptr_t opt = gmo_optimizer_new(GMO_RMSPROP, cfg, dims, ndims, 2, mm, device);
+        CHECK(opt != 0);
+        if (!opt) return;
+        for (int k = 0; k < 3; k++) {
+            const uintptr_t big = gmo_state_buffer(opt, kinds[k], 0), small = gmo_state_buffer(opt, kinds[k], 1);
+            CHECK(big != 0 && small != 0);
+            CHECK(cpu_device_requested_phase(big) == want[k]);
+            CHECK(cpu_device_requested_phase(small) == -1);
+            if (round == 0) first_handles[k] = big;
+            else CHECK(big == first_handles[k]);     // taken back from the pool of the same phase
+        }
+        gmo_cleanup(opt);
+        gmo_optimizer_free(opt);
+    }
+    const uintptr_t plain = gmo_allocate_buffer(mm, 1100 * 1024 * 4);
+    CHECK(plain != 0 && cpu_device_requested_phase(plain) == -1);
+    for (int k = 0; k < 3; k++) CHECK(plain != first_handles[k]);    // the plain pool is another pool
+    gmo_release_buffer(mm, plain);
+    CHECK(gm_allocate_buffer_phased(device, 1 << 21, 1, 100) == 0);          // not a multiple of 256
+    CHECK(gm_allocate_buffer_phased(device, 1 << 21, 1, 2 << 20) == 0);      // not below the period
+}
+
 static void json_documents()
 {
     // What encoding/json accepts and refuses, and nothing that strtod alone would let through.
@@ -388,6 +427,7 @@ int main()
     mixed_precision(device, mm);
     non_finite_state_is_refused(device, mm);
     pools_and_tensors(device, mm);
+    state_buffer_phases(device, mm);
     lbfgs(device, mm);
     schedulers();
     uintptr_t own = gmo_memory_manager_new(device);
