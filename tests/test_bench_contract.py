@@ -58,3 +58,21 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert "traffic" in roof and "not measured" in roof["traffic_source"]
     cpu = j["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+
+
+@pytest.mark.gpu
+def test_placement_workload_prints_both_placements_for_every_layout():
+    """The command behind profiles/adam_c5_1b_state_placement.md runs and reports the step with the state buffers
+    wherever the allocator puts them and at the optimizers' phases, in each layout of device memory."""
+    r = subprocess.run([sys.executable, BENCH, "--workload", "placement", "--steps", "2", "--warmup", "1"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    j = json.loads(lines[0])
+    assert len(j["layouts"]) == 6 and j["config"]["state_phases"] == [512 << 10, 1536 << 10]
+    for row in j["layouts"]:
+        for key in ("plain", "placed", "plain_again", "placed_again"):
+            assert 0.3 < row[key]["frac"] < 1.0, (row["spacer_bytes"], key, row[key])
+    assert j["plain_range"][0] <= j["plain_mean"] <= j["plain_range"][1]
+    assert j["placed_range"][0] <= j["placed_mean"] <= j["placed_range"][1]
