@@ -22,6 +22,7 @@ import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -29,9 +30,11 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
+sys.path.insert(0, os.path.join(ROOT, "go-metal_amd"))      # workloads.py: the configurations' tensor lists
 
 HBM_PEAK_GBS = 8000.0
+LINE_LIMIT = 1960         # bytes of the default run's final line: the driver keeps the tail of stdout
+ROTATE_C3 = 6            # copies of the 25M list stepped in turn by the default run: 6 x 300-400 MB
 STATE_PHASES = (512 << 10, 1536 << 10, 1 << 20)     # host/memory_manager.hpp, kStatePhases
 
 
@@ -95,6 +98,16 @@ WORKLOADS = {
 }
 
 
+def checker():
+    """The CPU oracle's Python binding (tests/oracle_lib.py).  Only the cpu_baseline legs call this: nothing on
+    the GPU path of this file imports from tests/ or touches the oracle."""
+    tests_dir = os.path.join(ROOT, "tests")
+    if tests_dir not in sys.path:
+        sys.path.insert(0, tests_dir)
+    from oracle_lib import oracle
+    return oracle()
+
+
 def cpu_model():
     """The host CPU's model name (reported beside the CPU baseline)."""
     try:
@@ -135,8 +148,7 @@ def per_launch_times(dev, launch, steps):
 
 def cpu_baseline_amp(sizes, hyper, grad_std, budget_params=96_000_000, target_seconds=3.0):
     """The oracle's mixed-precision Adam step (clean steps: check, unscale, update, fp16 copy) on this host."""
-    from oracle_lib import oracle
-    o = oracle()
+    o = checker()
     threads = min(16, os.cpu_count() or 1)
     chosen, total = [], 0
     for n in sizes:
@@ -172,9 +184,8 @@ def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_
     """The CPU oracle (a C port of the reference's update equations, OpenMP over elements) on
     this host, on the leading tensors of the same workload up to ~budget_params, for about
     target_seconds of CPU work."""
-    from oracle_lib import oracle
+    checker()
     from harness import OracleRun
-    oracle()
     threads = min(16, os.cpu_count() or 1)
     chosen, total = [], 0
     for n in sizes:
@@ -423,8 +434,7 @@ def bench_primitives(args, pkg, dev):
     if args.no_cpu_baseline:
         result["cpu_baseline"] = None
     else:
-        from oracle_lib import oracle
-        o = oracle()
+        o = checker()
         threads = min(16, os.cpu_count() or 1)
         sample = host
         o.f32_to_f16(sample, nthreads=threads)
@@ -446,8 +456,7 @@ def bench_primitives(args, pkg, dev):
 def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
     """The reference's algorithm as it runs it: one CPU thread, running fp32 sums
     (oracle/oracle_lbfgs.c in reference order), on the leading tensors of the workload."""
-    from oracle_lib import oracle
-    o = oracle()
+    o = checker()
     chosen, total = [], 0
     for k in sizes:
         if chosen and total + k > budget_params:
@@ -476,9 +485,79 @@ def lbfgs_cpu_baseline(sizes, m, budget_params=6_000_000, target_seconds=12.0):
 BASELINE_CONFIGS = ["c5", "c1", "c2-sgd", "c2-adam", "c3-rmsprop", "c3-adagrad", "c3-adadelta", "c3-nadam", "c4"]
 
 
+def _sig(x, digits=5):
+    """A number with `digits` significant digits (the final line is kept short; full precision is in the file);
+    an integer where that loses nothing, which prints shorter."""
+    if x is None or isinstance(x, (str, bool)) or x == 0:
+        return x
+    r = float(f"{x:.{digits}g}")
+    return int(r) if abs(r) >= 10 ** digits else r
+
+
+def compact_line(results, records_file):
+    """The one line the default run prints LAST, under 2 KB: the headline configuration's record (config 5, fp32
+    Adam) with its roofline and CPU baseline, the two forms of the mixed-precision step over the same list, and per
+    other configuration only the figures (ms per step, params/s, fraction of peak, kernel ms, CPU params/s).  The
+    full per-configuration records, prose fields included, are in `records_file`."""
+    h = results["c5"]
+    roof = h["roofline"]
+    line = {
+        "metric": h["metric"], "value": _sig(h["value"], 7), "unit": h["unit"], "n_gpus": 1, "steps": h["steps"],
+        "warmup": h["warmup"], "ms_per_step": _sig(h["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": h["config"]["workload"], "tensors": h["config"]["tensors"], "params": h["config"]["params"]},
+        "roofline": {"bound": "hbm", "achieved": _sig(roof["achieved"], 6), "peak": roof["peak"], "unit": "GB/s",
+                     "frac": _sig(roof["frac"]), "traffic": roof.get("traffic"), "kernel": roof["kernel"],
+                     "kernel_ms": _sig(roof["kernel_ms"], 6), "bytes_per_param": roof["bytes_per_param"]},
+    }
+    cpu = h.get("cpu_baseline")
+    line["cpu_baseline"] = None if cpu is None else {
+        "value": _sig(cpu["value"]), "unit": cpu["unit"], "cores": cpu["cores"], "kind": cpu["kind"],
+        "sample": cpu["sample"][:64]}
+    amp = h.get("amp")
+    if amp:
+        form = lambda r: {"frac": _sig(r["roofline"]["frac"], 4), "ms_per_step": _sig(r["ms_per_step"], 4)}
+        line["amp"] = {"default": amp["default_form"], "one_pass": form(amp["one_pass"]), "in_place": form(amp["in_place"]),
+                       "bytes_per_param": 28}
+    configs = {}
+    for name, r in results.items():
+        if name == "c5":
+            continue
+        rr = r.get("roofline") or {}
+        c = {"ms_per_step": _sig(r.get("ms_per_step"), 4), "steps": r.get("steps"), "value": _sig(r.get("value"), 4),
+             "frac": _sig(rr.get("frac"), 4), "kernel_ms": _sig(rr.get("kernel_ms"), 4)}
+        if rr.get("frac_hbm") is not None:
+            c["frac_hbm"] = _sig(rr["frac_hbm"], 4)
+        if r.get("one_pass"):
+            c["frac_one_pass"] = _sig(r["one_pass"]["roofline"]["frac"], 4)
+        cb = r.get("cpu_baseline")
+        c["cpu"] = _sig(cb["value"], 3) if cb else None
+        configs[name] = c
+    line["configs"] = configs
+    line["records"] = records_file
+
+    def render():
+        text = json.dumps(line, separators=(",", ":"))
+        # integers that end in six or more zeros in exponent form: 235100000000 -> 2351e8 (the same JSON number)
+        return re.sub(r"(?<=[:\[,])(\d+?)(0{6,})(?=[,}\]])", lambda m: f"{m.group(1)}e{len(m.group(2))}", text)
+
+    # the limit holds by construction: if the figures print longer than expected, the least needed fields go
+    def shorten_sample():
+        if line["cpu_baseline"]:
+            line["cpu_baseline"]["sample"] = line["cpu_baseline"]["sample"][:24]
+    trims = [shorten_sample] + [lambda key=key: [c.pop(key, None) for c in configs.values()]
+                                for key in ("kernel_ms", "steps", "cpu")]
+    text = render()
+    while len(text) > LINE_LIMIT and trims:
+        trims.pop(0)()
+        text = render()
+    return text
+
+
 def run_children(args, names):
     """Each named workload as a child process, started before this process has made any GPU call (it never
-    makes one).  The line printed is the headline configuration's, with the others under "configs"."""
+    makes one).  The full records go to gpurun_out/bench_configs.json; the last line printed is the headline
+    configuration's, with the other configurations' figures under "configs" (compact_line)."""
     import subprocess
     results = {}
     for name in names:
@@ -492,14 +571,19 @@ def run_children(args, names):
         steps = args.steps if headline or name == "lbfgs-c3" else max(args.steps, 200)
         cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", str(steps),
                "--warmup", str(warmup), "--cpu-seconds", str(args.cpu_seconds if name == "c5" else min(args.cpu_seconds, 3.0))]
+        if name.startswith("c3-"):
+            cmd += ["--rotate", str(ROTATE_C3)]
         if args.no_cpu_baseline:
             cmd.append("--no-cpu-baseline")
         print(f"running {name}", file=sys.stderr, flush=True)
         out = subprocess.run(cmd, check=True, stdout=subprocess.PIPE, text=True).stdout
         results[name] = json.loads(out.strip().splitlines()[-1])
-    headline = dict(results["c5"])
-    headline["configs"] = {k: v for k, v in results.items() if k != "c5"}
-    print(json.dumps(headline))
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    os.makedirs(out_dir, exist_ok=True)
+    records_file = os.path.join("gpurun_out", "bench_configs.json")
+    with open(os.path.join(ROOT, records_file), "w") as f:
+        json.dump(results, f, indent=1)
+    print(compact_line(results, records_file), flush=True)
 
 
 def main():
@@ -516,6 +600,9 @@ def main():
                     "'NT,REV' with NT 1/0 = non-temporal loads on/off and REV 1/0 = walk the table backwards")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-amp", action="store_true")
+    ap.add_argument("--rotate", type=int, default=0,
+                    help="also step K independent copies of the list in turn (K x footprint beyond the 256 MB memory-side "
+                         "cache), so that no stream of a step is still cached from the step before: roofline.frac_hbm")
     ap.add_argument("--history", type=int, default=0, help="L-BFGS workloads: history size (default 10)")
     ap.add_argument("--rule", default="", choices=["", "sgd", "adam", "rmsprop", "adagrad", "adadelta", "nadam"],
                     help="run another update rule (with the benchmark configurations' hyper-parameters for it) over the workload's list")
@@ -607,8 +694,36 @@ def main():
     bpp = BYTES_PER_PARAM[rule]
     achieved = params * bpp / (event_ms * 1e-3) / 1e9
 
-    # measured ceiling: plain 16-byte copy kernel, same box, same run
-    probe_bytes = min(1 << 30, max(1 << 24, (4 * max(sizes)) // 16 * 16))
+    # ---- the same step over K independent copies of the list in turn: an HBM figure for lists that would
+    # otherwise stay (partly) in the 256 MB memory-side cache from one step to the next ----
+    rotated = None
+    if args.rotate > 1:
+        copies = [(cw, cg, cs)]
+        for c in range(1, args.rotate):
+            w2 = [dev.alloc(4 * s) for s in sizes]
+            g2 = [dev.alloc(4 * s) for s in sizes]
+            st2 = [[dev.alloc(4 * s, zero=True, phase=state_phase(j, 4 * s)) for s in sizes] for j in range(nstate)]
+            for k, s in enumerate(sizes):
+                lib.gm_fill_normal_f32(D, w2[k], s, 0x6D657461 + k + 7919 * c, 0.0, 0.02)
+                lib.gm_fill_normal_f32(D, g2[k], s, 0x12345 + k + 7919 * c, 0.0, grad_std)
+            copies.append((pkg.handle_array(w2), pkg.handle_array(g2), [pkg.handle_array(x) for x in st2]))
+        dev.synchronize()
+        turn = {"i": 0}
+
+        def launch_rotating():
+            nonlocal cw, cg, cs
+            cw, cg, cs = copies[turn["i"] % len(copies)]
+            turn["i"] += 1
+            launch_fp32()
+
+        rot_steps = -(-args.steps // len(copies)) * len(copies)       # every copy the same number of times
+        rot_wall, rot_event = time_steps(dev, launch_rotating, rot_steps, max(args.warmup, len(copies)))
+        cw, cg, cs = copies[0]
+        rotated = {"copies": len(copies), "steps": rot_steps, "ms_per_step": rot_wall, "kernel_ms": rot_event,
+                   "footprint_bytes": len(copies) * params * 4 * (2 + nstate)}
+
+    # measured ceiling: plain 16-byte copy kernel over 1 GiB (an HBM figure whatever the workload's size), same run
+    probe_bytes = 1 << 30
     src, dst = dev.alloc(probe_bytes), dev.alloc(probe_bytes)
     _, copy_ms = time_steps(dev, lambda: lib.gm_copy_probe(D, dst, src, probe_bytes), 10, 3)
     copy_gbs = 2 * probe_bytes / (copy_ms * 1e-3) / 1e9
@@ -637,10 +752,20 @@ def main():
     result["config"]["state_placement"] = ("state buffers of more than 4 MiB start at phases of their own modulo 2 MiB, "
                                             "as the optimizers allocate them: " + ", ".join(str(p) for p in STATE_PHASES[:nstate]))
     footprint = params * 4 * (2 + nstate)            # every stream of the step, in bytes
+    result["roofline"]["footprint_bytes"] = footprint
+    if rotated:
+        hbm = params * bpp / (rotated["kernel_ms"] * 1e-3) / 1e9
+        result["roofline"].update({"frac_hbm": hbm / HBM_PEAK_GBS, "achieved_hbm": hbm, "rotated": rotated,
+                                   "frac_of_copy_kernel": hbm / copy_gbs})
     if footprint < 256 * 1024 * 1024:
         result["roofline"]["note"] = (f"the step's {footprint / 1e6:.0f} MB stay in the 256 MB memory-side cache between "
                                       "steps and the kernel is a few microseconds of launch latency: 'achieved' counts "
                                       "algorithmic bytes per second, it is not an HBM figure for this workload")
+    elif footprint < 1 << 30:
+        result["roofline"]["note"] = (f"the step's {footprint / 1e6:.0f} MB are of the order of the 256 MB memory-side "
+                                      "cache, which serves part of every step from what the step before left there: 'frac' "
+                                      "is faster than HBM alone would allow; 'frac_hbm' (--rotate: independent copies of "
+                                      "the list stepped in turn) is the HBM figure")
 
     # ---- mixed-precision Adam on the same list (fp16 gradients, fp16 weight copy) ----
     if rule == "adam" and not args.no_amp:
@@ -744,16 +869,15 @@ def main():
                       "max_steps_in_flight": lib.gm_amp_state_max_in_flight(amp2)},
         }
         lib.gm_amp_state_destroy(amp2)
-        # The one-pass form leads the record (unscale, check, skip and loss-scale update in the update pass);
-        # the in-place form, which keeps one set of state and reads the gradients twice, sits beside it.
+        # StepAMP runs the in-place form unless the caller asked for ping-pong state (EnablePingPong): the in-place
+        # form keeps the caller's own fp32 weight buffers current after every step, the one-pass form does not.
         in_place = result["amp"]
-        lead = in_place.pop("one_pass")
-        lead["dtype"] = in_place["dtype"]
-        lead["form"] = ("one pass over ping-pong state: weights and moments kept twice (+12 B/param of HBM), "
-                        "execute_adam_amp_step_fused / EnablePingPong")
+        one_pass = in_place.pop("one_pass")
+        one_pass["dtype"] = in_place["dtype"]
+        one_pass["form"] = ("one pass over ping-pong state: weights and moments kept twice (+12 B/param of HBM), "
+                            "execute_adam_amp_step_fused / EnablePingPong")
         in_place["form"] = "in place: one set of state, the gradients read twice (execute_adam_amp_step, the default of StepAMP)"
-        lead["in_place"] = in_place
-        result["amp"] = lead
+        result["amp"] = {"default_form": "in_place", "in_place": in_place, "one_pass": one_pass}
         if not args.no_cpu_baseline and args.workload in ("c4", "c5"):
             result["amp"]["cpu_baseline"] = cpu_baseline_amp(sizes, hyper, grad_std, target_seconds=min(args.cpu_seconds, 3.0))
 
@@ -763,16 +887,18 @@ def main():
         result["cpu_baseline"] = None
 
     if args.workload == "c4" and "amp" in result:
-        # configuration 4 IS the mixed-precision step: its figures lead, the fp32 step over the same list follows
+        # configuration 4 IS the mixed-precision step: the form StepAMP runs by default leads, the one-pass form and
+        # the fp32 step over the same list follow
         amp_part = result.pop("amp")
+        lead = amp_part[amp_part["default_form"]]
         fp32_part = {k: result[k] for k in ("value", "unit", "ms_per_step", "dtype", "roofline", "cpu_baseline")}
         result.update({"metric": "params updated/sec (mixed-precision Adam step, fp16 gradients and weight copy) + "
                                  "achieved HBM GB/s (% of peak)",
-                       "value": amp_part["value"], "ms_per_step": amp_part["ms_per_step"], "dtype": amp_part["dtype"],
-                       "roofline": amp_part["roofline"], "cpu_baseline": amp_part.get("cpu_baseline"),
-                       "skipped_steps": amp_part["skipped_steps"], "async": amp_part["async"],
-                       "form": amp_part["form"], "entry_point": amp_part["entry_point"],
-                       "in_place": amp_part["in_place"], "fp32_adam": fp32_part})
+                       "value": lead["value"], "ms_per_step": lead["ms_per_step"], "dtype": lead["dtype"],
+                       "roofline": lead["roofline"], "cpu_baseline": amp_part.get("cpu_baseline"),
+                       "skipped_steps": lead["skipped_steps"], "async": lead["async"],
+                       "form": lead["form"], "default_form": amp_part["default_form"],
+                       "in_place": amp_part["in_place"], "one_pass": amp_part["one_pass"], "fp32_adam": fp32_part})
 
     dev.close()
     print(json.dumps(result))

@@ -1,4 +1,4 @@
-"""Tensor lists of the five benchmark configurations (shared by the parity tests and bench.py)."""
+"""Tensor lists of the five benchmark configurations (product configuration: bench.py measures them, the parity tests step them)."""
 import numpy as np
 
 # config 2: conv [oc, ic, k, k] + bias, BatchNorm gamma / beta, dense [in, out] + bias
