@@ -75,6 +75,7 @@ ABI = {
     "execute_adam_amp_step_fused": (i, [u, up, up, up, up, up, up, up, up, i, ip, f, f, f, f, f, i, u, ip, fp, ip, ip]),
     "execute_adam_amp_step_fused_async": (i, [u, up, up, up, up, up, up, up, up, i, ip, f, f, f, f, f, u]),
     "gm_amp_state_current_set": (i, [u]),
+    "gm_amp_state_set_current_set": (i, [u, i]),
     "gm_timer_start": (i, [u]),
     "gm_timer_stop": (f, [u]),
     "gm_fill_normal_f32": (i, [u, u, ctypes.c_size_t, ctypes.c_uint64, f, f]),

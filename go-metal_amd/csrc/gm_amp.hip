@@ -7,7 +7,7 @@
 // in place (execute_adam_amp_step[_async]): weights and moments are updated where they lie, so
 //   nothing may be written before every gradient has been checked: a check launch reads the fp16
 //   gradients, an update launch reads them again (30 bytes move per parameter for 28 algorithmic
-//   ones), a one-lane epilogue advances the loss-scale state.
+//   ones); one lane of the update launch advances the loss-scale state.
 // ping-pong (execute_adam_amp_step_fused[_async]): weights and moments exist twice (sets A and B),
 //   one of them current.  ONE launch reads the current set and the gradients, checks the
 //   gradients as it goes, and writes the other set; the epilogue makes that set current only if
@@ -15,6 +15,12 @@
 //   never written: every stream moves once, 28 bytes per parameter.  The fp16 weight copy has a
 //   single consumer-visible buffer and is written speculatively; after a dropped step a repair
 //   pass (which returns at once after an applied one) rewrites it from the current weights.
+//
+// The loss-scale state lives in HBM as two records and an overflow word.  A step reads one record
+// (its pre-state) and one lane writes the advanced state into the other, which the next step
+// reads: no kernel reads a record that the same launch writes.  The overflow word holds the
+// stamp of the last step that saw an inf / NaN; every step carries its own 64-bit stamp, so the
+// word needs no clearing and means "this step overflowed" only while it equals this step's stamp.
 #include "gm_launch.hpp"
 #include "gm_update_kernels.hpp"
 
@@ -33,9 +39,7 @@ struct alignas(16) AmpDeviceState {
     // head: the 16 bytes every workgroup of the update kernel reads with one scalar load
     int current_set;        // ping-pong step: 0 = set A holds the current weights and moments, 1 = set B
     float inv_scale;        // 1.0f / scale, kept by whoever changes scale (IEEE division on host and device alike)
-    unsigned int found_inf; // the stamp of the step whose gradients held an inf / NaN (every step carries its own
-                            // non-zero stamp, so the word needs no clearing between the kernels of a step: it means
-                            // "this step overflowed" only while it equals this step's stamp)
+    int unused;
     int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
     // tail
     float scale;
@@ -48,6 +52,15 @@ struct alignas(16) AmpDeviceState {
     int pad;
 };
 static_assert(sizeof(AmpDeviceState) == 48, "AmpDeviceState layout");
+
+// What a loss-scale state keeps on the device: the record the next step reads and the record it
+// writes (they swap roles with every step), and the stamp of the last step that overflowed.
+struct alignas(16) AmpDeviceBlock {
+    AmpDeviceState slot[2];
+    unsigned long long overflow;
+    unsigned long long pad;
+};
+static_assert(sizeof(AmpDeviceBlock) == 112, "AmpDeviceBlock layout");
 
 // Bias corrections for the asynchronous step.  The host does not know how many of the steps
 // still in flight were applied, so it sends the corrections (glibc powf, like every other
@@ -65,8 +78,8 @@ struct AmpBiasTable {
 // one store of the step's stamp per workgroup that saw a hit.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
-amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__restrict__ state, int reverse,
-                          unsigned int stamp)
+amp_overflow_check_kernel(const Chunk *__restrict__ chunks, unsigned long long *__restrict__ overflow, int reverse,
+                          unsigned long long stamp)
 {
     __shared__ unsigned int wave_hit[kBlock / 64];
     // reverse: the table is walked from its end, so that the check finishes on the gradients the
@@ -106,8 +119,42 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, AmpDeviceState *__re
         unsigned int any = 0;
 #pragma unroll
         for (int k = 0; k < kBlock / 64; k++) any |= wave_hit[k];
-        if (any) __hip_atomic_store(&state->found_inf, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (any) __hip_atomic_store(overflow, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+}
+
+// Advances the loss-scale state machine after a step (one lane): reads the step's pre-state and
+// writes its post-state into the record the next step reads.  found: this step's gradients held
+// an inf / NaN.
+__device__ inline void amp_advance(const AmpDeviceState *pre, AmpDeviceState *post, AmpDeviceState *host_mirror,
+                                   bool found, int ping_pong)
+{
+    AmpDeviceState st = *pre;
+    // The scale stays a normal, finite fp32 number whatever the run does: a growth that would
+    // overflow to infinity (about 112 uninterrupted growth intervals from 65536) and a backoff
+    // that would leave the normal range are not applied.  Unbounded, the scale would stick at
+    // +inf (inf * 0.5 = inf) with a reciprocal of 0, or reach 0 with a reciprocal of +inf.
+    if (found) {
+        const float next = st.scale * st.backoff_factor;
+        if (next >= kMinLossScale) st.scale = next;
+        st.growth_tracker = 0;
+        st.skipped_steps += 1;
+    } else {
+        st.applied_steps += 1;
+        if (ping_pong) st.current_set ^= 1;      // the set just written is the current one from here on
+        st.growth_tracker += 1;
+        if (st.growth_tracker == st.growth_interval) {
+            const float next = st.scale * st.growth_factor;
+            if (next <= kMaxLossScale) st.scale = next;
+            st.growth_tracker = 0;
+        }
+    }
+    st.inv_scale = 1.0f / st.scale;
+    st.last_skipped = found ? 1 : 0;
+    *post = st;
+    // The post-state also goes straight into pinned host memory: the host reads it once the
+    // stream (or the event recorded after this launch) has completed, without a copy launch.
+    if (host_mirror) *host_mirror = st;
 }
 
 // The bias corrections of the step count the device has reached: entry (applied - base) of the
@@ -121,22 +168,29 @@ __device__ inline void amp_pick_bias(StepParams &prm, const AmpBiasTable &bias, 
     prm.bc2 = bias.bc2[pick];
 }
 
-// Phase B: the Adam update on unscaled gradients, skipped as a whole when the
-// check stored this step's stamp.
+// Phase B: the Adam update on unscaled gradients, skipped as a whole when the check stored this
+// step's stamp.  The launch also carries the step's epilogue: with `post` set, lane 0 of workgroup
+// 0 advances the loss-scale state from the pre-state into the other record (the check has
+// finished, so every workgroup of this launch sees the same decision; nothing it reads is written
+// while it runs).
 template <int VEC, bool NT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, StepParams prm,
-                       const AmpDeviceState *__restrict__ state, AmpBiasTable bias, unsigned int stamp)
+                       const AmpDeviceState *__restrict__ pre, const unsigned long long *__restrict__ overflow,
+                       AmpBiasTable bias, unsigned long long stamp, AmpDeviceState *post, AmpDeviceState *host_mirror)
 {
-    // The state's head (current set, reciprocal of the scale, overflow stamp, applied steps) comes with one 16-byte scalar load
-    // and the chunk descriptor with another, both issued before anything is decided; the bias
-    // table sits in the kernel arguments and its entry comes with an indexed scalar load.
-    const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
+    // The pre-state's head (current set, reciprocal of the scale, applied steps) comes with one 16-byte scalar load,
+    // the overflow word with another and the chunk descriptor with a third, all issued before anything is decided;
+    // the bias table sits in the kernel arguments and its entry comes with an indexed scalar load.
+    const uintx4 head = *reinterpret_cast<const uintx4 *>(pre);
+    const unsigned long long seen = *overflow;
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
     const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
+    const bool found = seen == stamp;
+    if (post != nullptr && blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 0);
     // (the weight pointer is never null; testing it here makes the compiler fetch the whole
     // descriptor before the branch instead of the count first and the addresses after it)
-    if ((head.z == stamp) | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
+    if (found | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
         return;                                                        // step dropped, or an idle slice
     const float inv_scale = __uint_as_float(head.y);
     amp_pick_bias(prm, bias, (int)head.w);
@@ -199,18 +253,19 @@ __device__ inline bool amp_fused_finish(const FusedLoaded<N> &x, const Chunk &ou
 // The ping-pong step: one pass.  Reads weights and moments of the current set and the fp16
 // gradients, writes the other set and the fp16 weight copy, and stores the step's stamp when a
 // gradient of its own is +-inf or NaN.  Its arithmetic never looks at the stamp: what it writes
-// becomes current only if the epilogue finds that no workgroup stored it.
+// becomes current only if the epilogue finds that no workgroup stored it.  (The overflow word is
+// accessed with atomic loads and stores only while this launch runs; the pre-state is read-only.)
 // (The state pointer is the first argument and the early exit tests the head: both make the
 // compiler fetch the state's head together with the two descriptors, straight after the kernel
 // arguments, instead of behind the first branch; that shortens the chain of dependent scalar
 // loads in front of the first global load from four to two.)
 template <int VEC, bool NT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
-amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restrict__ set_a,
+amp_adam_fused_kernel(const AmpDeviceState *__restrict__ pre, const Chunk *__restrict__ set_a,
                       const Chunk *__restrict__ set_b, uint32_t slice_shift, StepParams prm, AmpBiasTable bias,
-                      unsigned int stamp)
+                      unsigned long long stamp, unsigned long long *__restrict__ overflow)
 {
-    const uintx4 head = *reinterpret_cast<const uintx4 *>(state);
+    const uintx4 head = *reinterpret_cast<const uintx4 *>(pre);
     const uint32_t c = blockIdx.x >> slice_shift;
     const Chunk a = set_a[c];
     const Chunk b = set_b[c];
@@ -243,70 +298,34 @@ amp_adam_fused_kernel(AmpDeviceState *__restrict__ state, const Chunk *__restric
     // inf would otherwise send millions of stores to one address).  Every writer stores the same value.
     const unsigned long long hit = __ballot(bad);
     if (hit != 0ull && (threadIdx.x & 63u) == (unsigned int)(__ffsll((long long)hit) - 1) &&
-        __hip_atomic_load(&state->found_inf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stamp)
-        __hip_atomic_store(&state->found_inf, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_load(overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stamp)
+        __hip_atomic_store(overflow, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Advances the loss-scale state machine after a step (one lane).  found: this step's gradients held
-// an inf / NaN.  The stamp word is left alone while it names this step and zeroed otherwise, so a
-// stale stamp can never meet its own value again when the 32-bit stamp counter wraps.
-__device__ inline void amp_advance(AmpDeviceState *state, AmpDeviceState *host_mirror, bool found, unsigned int stamp,
-                                   int ping_pong)
-{
-    AmpDeviceState st = *state;
-    // The scale stays a normal, finite fp32 number whatever the run does: a growth that would
-    // overflow to infinity (about 112 uninterrupted growth intervals from 65536) and a backoff
-    // that would leave the normal range are not applied.  Unbounded, the scale would stick at
-    // +inf (inf * 0.5 = inf) with a reciprocal of 0, or reach 0 with a reciprocal of +inf.
-    if (found) {
-        const float next = st.scale * st.backoff_factor;
-        if (next >= kMinLossScale) st.scale = next;
-        st.growth_tracker = 0;
-        st.skipped_steps += 1;
-    } else {
-        st.applied_steps += 1;
-        if (ping_pong) st.current_set ^= 1;      // the set just written is the current one from here on
-        st.growth_tracker += 1;
-        if (st.growth_tracker == st.growth_interval) {
-            const float next = st.scale * st.growth_factor;
-            if (next <= kMaxLossScale) st.scale = next;
-            st.growth_tracker = 0;
-        }
-    }
-    st.inv_scale = 1.0f / st.scale;
-    st.last_skipped = found ? 1 : 0;
-    st.found_inf = found ? stamp : 0u;
-    *state = st;
-    // The post-state also goes straight into pinned host memory: the host reads it once the
-    // stream (or the event recorded after this launch) has completed, without a copy launch.
-    if (host_mirror) *host_mirror = st;
-}
-
-// Epilogue of the in-place step (one lane, same stream, after the update pass has drained).  A
-// separate launch rather than a last-workgroup ticket: a single counter bumped by every workgroup
-// of a 250k-workgroup grid serialises in the memory-side atomic unit.
-__global__ void amp_finalize_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror, unsigned int stamp)
+// Epilogue of a step over an empty list (one lane): there is no update launch to carry it.
+__global__ void amp_finalize_kernel(const AmpDeviceState *pre, AmpDeviceState *post, AmpDeviceState *host_mirror,
+                                    const unsigned long long *overflow, unsigned long long stamp, int ping_pong)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    amp_advance(state, host_mirror, state->found_inf == stamp, stamp, 0);
+    amp_advance(pre, post, host_mirror, *overflow == stamp, ping_pong);
 }
 
 // Epilogue of the ping-pong step, and the repair of the fp16 weight copy, in one launch.  After a
 // dropped step the copy holds what the discarded update wrote: it is rewritten from the current
 // weights (the copy of an applied step is half(w) by construction, so this restores it bit for
 // bit).  Small fixed grid; after an applied step every workgroup returns on its first load.
-// Lane 0 of workgroup 0 advances the state machine while the other workgroups read two words of
-// the same record; that is safe because whatever those readers act on does not change under them:
-// the stamp word either keeps naming this step (dropped: they repair, and the current set is not
-// flipped) or goes from one value that is not this step's stamp to another (applied: they return).
+// Lane 0 of workgroup 0 writes the advanced state into the record the next step reads; what the
+// workgroups of this launch read (the overflow word, the current set of the pre-state) is
+// written by nobody while it runs.
 __global__ void __launch_bounds__(kBlock)
-amp_finalize_repair_kernel(AmpDeviceState *state, AmpDeviceState *host_mirror, unsigned int stamp,
+amp_finalize_repair_kernel(const AmpDeviceState *pre, AmpDeviceState *post, AmpDeviceState *host_mirror,
+                           const unsigned long long *overflow, unsigned long long stamp,
                            const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t num_chunks)
 {
-    const bool found = __hip_atomic_load(&state->found_inf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == stamp;
-    if (blockIdx.x == 0 && threadIdx.x == 0) amp_advance(state, host_mirror, found, stamp, 1);
+    const bool found = *overflow == stamp;
+    if (blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 1);
     if (!found) return;
-    const Chunk *current = __hip_atomic_load(&state->current_set, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ? set_b : set_a;
+    const Chunk *current = pre->current_set != 0 ? set_b : set_a;      // a dropped step keeps the current set
     for (uint32_t c = blockIdx.x; c < num_chunks; c += gridDim.x) {
         const Chunk ch = current[c];
         if (ch.p[kSlotWeight16] == nullptr) continue;
@@ -326,7 +345,8 @@ extern "C" {
 struct AmpState {
     uint64_t magic;
     Context *ctx;
-    AmpDeviceState *d_state;
+    AmpDeviceBlock *d_block;
+    int slot;                            // which record of d_block the next step reads (the state as of now)
     AmpDeviceState *h_pinned;            // kAmpMaxInFlight + 1 slots: [0] synchronous read-backs, [1..] the ring
     hipEvent_t ring_event[kAmpMaxInFlight];
     // asynchronous steps: issue numbers count execute_adam_amp_step_async calls
@@ -334,7 +354,7 @@ struct AmpState {
     uint64_t confirmed_issue;            // newest step whose post-state the host has seen
     int confirmed_applied;               // the device's applied_steps after that step
     int max_in_flight;                   // deepest run-ahead seen (diagnostics)
-    unsigned int last_stamp;             // stamp of the newest step issued (either form); never 0
+    unsigned long long last_stamp;       // stamp of the newest step issued (either form); never 0, never repeats
 };
 static const uint64_t kAmpMagic = 0x676D5F616D705F73ull;   // "gm_amp_s"
 
@@ -347,7 +367,7 @@ static AmpState *amp_from_handle(uintptr_t h)
 
 static bool amp_upload(AmpState *s)
 {
-    return hip_ok(hipMemcpyAsync(s->d_state, s->h_pinned, sizeof(AmpDeviceState),
+    return hip_ok(hipMemcpyAsync(&s->d_block->slot[s->slot], s->h_pinned, sizeof(AmpDeviceState),
                                  hipMemcpyHostToDevice, s->ctx->stream), "amp state upload") &&
            hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize");
 }
@@ -355,7 +375,7 @@ static bool amp_upload(AmpState *s)
 // Waits for everything on the stream and reads the state back: afterwards no step is in flight.
 static bool amp_download(AmpState *s)
 {
-    if (!hip_ok(hipMemcpyAsync(s->h_pinned, s->d_state, sizeof(AmpDeviceState),
+    if (!hip_ok(hipMemcpyAsync(s->h_pinned, &s->d_block->slot[s->slot], sizeof(AmpDeviceState),
                                hipMemcpyDeviceToHost, s->ctx->stream), "amp state download") ||
         !hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize"))
         return false;
@@ -390,7 +410,7 @@ static bool amp_poll(AmpState *s, bool must_free_slot)
 
 static void amp_free(AmpState *s)
 {
-    if (s->d_state) (void)hipFree(s->d_state);
+    if (s->d_block) (void)hipFree(s->d_block);
     if (s->h_pinned) (void)hipHostFree(s->h_pinned);
     for (hipEvent_t e : s->ring_event)
         if (e) (void)hipEventDestroy(e);
@@ -418,7 +438,8 @@ try {
     auto *s = new AmpState{};
     s->magic = kAmpMagic;
     s->ctx = ctx;
-    bool ok = hip_ok(hipMalloc(&s->d_state, sizeof(AmpDeviceState)), "hipMalloc(amp state)") &&
+    bool ok = hip_ok(hipMalloc(&s->d_block, sizeof(AmpDeviceBlock)), "hipMalloc(amp state)") &&
+              hip_ok(hipMemsetAsync(s->d_block, 0, sizeof(AmpDeviceBlock), ctx->stream), "hipMemsetAsync(amp state)") &&
               hip_ok(hipHostMalloc(&s->h_pinned, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState),
                                    hipHostMallocDefault), "hipHostMalloc(amp state)");
     for (int k = 0; ok && k < kAmpMaxInFlight; k++)
@@ -516,11 +537,19 @@ try {
     return -6;
 }
 
-// The next step's stamp (the context lock is held).
-static unsigned int amp_next_stamp(AmpState *amp)
+// The next step's stamp (the context lock is held).  64 bits: it does not come round again.
+static unsigned long long amp_next_stamp(AmpState *amp)
 {
-    if (++amp->last_stamp == 0u) ++amp->last_stamp;
-    return amp->last_stamp;
+    return ++amp->last_stamp;
+}
+
+// The records of the step about to be enqueued: it reads `pre` and writes `post`, which the step
+// after it reads (the context lock is held).
+static void amp_take_records(AmpState *amp, AmpDeviceState *&pre, AmpDeviceState *&post)
+{
+    pre = &amp->d_block->slot[amp->slot];
+    post = &amp->d_block->slot[amp->slot ^ 1];
+    amp->slot ^= 1;
 }
 
 static StepParams amp_step_params(float learning_rate, float beta1, float beta2, float epsilon, float weight_decay)
@@ -579,7 +608,8 @@ static PlanRequest amp_request(uintptr_t *weight_buffers, uintptr_t *gradient16_
     return req;
 }
 
-// Plan, parameters and the three launches shared by the synchronous and the asynchronous in-place step.
+// Plan, parameters and the launches (check, update with the epilogue) shared by the synchronous and the
+// asynchronous in-place step.
 static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffers,
                        uintptr_t *gradient16_buffers, uintptr_t *momentum_buffers,
                        uintptr_t *variance_buffers, uintptr_t *weight16_buffers, int num_weights,
@@ -595,41 +625,49 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
         return -16;
     }
     const StepParams p = amp_step_params(learning_rate, beta1, beta2, epsilon, weight_decay);
+    const uint32_t chunks = l.plan->num_chunks;
+    hipStream_t st = l.ctx->stream;
+    int vec = current_vec(l.ctx);
+    if (vec == 0) vec = auto_vec(8);
+    const bool nt = current_nontemporal(l.ctx);
+    int block = current_block(l.ctx);
+    if (block == 0) block = auto_block(8);
+    SegmentLaunch seg[2];
+    int count = 0;
+    if (chunks > 0 && !launch_geometry(*l.plan, vec, block, seg, count)) return -6;
+    // nothing below fails before the launches: the step takes its stamp and its two records
     AmpDeviceState *host_mirror;
     AmpBiasTable bias;
     if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
-    const unsigned int stamp = amp_next_stamp(amp);
+    const unsigned long long stamp = amp_next_stamp(amp);
+    AmpDeviceState *pre, *post;
+    amp_take_records(amp, pre, post);
+    unsigned long long *overflow = &amp->d_block->overflow;
 
-    const uint32_t chunks = l.plan->num_chunks;
-    hipStream_t st = l.ctx->stream;
     if (chunks > 0) {
-        int vec = current_vec(l.ctx);
-        if (vec == 0) vec = auto_vec(8);
-        const bool nt = current_nontemporal(l.ctx);
-        int block = current_block(l.ctx);
-        if (block == 0) block = auto_block(8);
-        SegmentLaunch seg[2];
-        int count;
-        if (!launch_geometry(*l.plan, vec, block, seg, count)) return -6;
         // the check walks the whole table, one workgroup per chunk of either segment
         const int reverse = l.ctx->amp_check_reverse.load();
         if (nt && l.ctx->amp_check_nontemporal.load())
-            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse, stamp);
+            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, overflow, reverse, stamp);
         else
-            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, amp->d_state, reverse, stamp);
-#define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, amp->d_state, bias, stamp)
+            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, overflow, reverse, stamp);
+        // the last update launch of the step carries the epilogue (the earlier one reads the same pre-state)
+#define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, pre, overflow, bias, stamp, \
+                                                                                 last ? post : nullptr, last ? host_mirror : nullptr)
 #define GM_LAUNCH_AMP_B(B)                                                              \
         if (vec == 4) { if (nt) GM_LAUNCH_AMP(4, true, B); else GM_LAUNCH_AMP(4, false, B); }        \
         else if (vec == 2) { if (nt) GM_LAUNCH_AMP(2, true, B); else GM_LAUNCH_AMP(2, false, B); }   \
         else { if (nt) GM_LAUNCH_AMP(1, true, B); else GM_LAUNCH_AMP(1, false, B); }
         for (int s = 0; s < count; s++) {
             const SegmentLaunch &g = seg[s];
+            const bool last = s == count - 1;
             if (block == 128) { GM_LAUNCH_AMP_B(128) } else { GM_LAUNCH_AMP_B(kBlock) }
         }
 #undef GM_LAUNCH_AMP_B
 #undef GM_LAUNCH_AMP
+    } else {
+        amp_finalize_kernel<<<1, 64, 0, st>>>(pre, post, host_mirror, overflow, stamp, 0);
     }
-    amp_finalize_kernel<<<1, 64, 0, st>>>(amp->d_state, host_mirror, stamp);
     return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
 }
 
@@ -670,8 +708,9 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
         plan_a->segment[0].num_chunks != plan_b->segment[0].num_chunks ||
         plan_a->segment[0].chunk_elements != plan_b->segment[0].chunk_elements ||
         plan_a->segment[1].chunk_elements != plan_b->segment[1].chunk_elements ||
-        plan_a->total_elements != plan_b->total_elements) {
-        // only a tensor skipped in one set and not the other (a buffer shorter than its size) gets here
+        plan_a->total_elements != plan_b->total_elements || plan_a->kept_signature != plan_b->kept_signature) {
+        // only a tensor skipped in one set and not the other (a buffer shorter than its size) gets here: chunk c of
+        // set A must be the same tensor and range as chunk c of set B
         set_error("sets A and B do not hold the same tensors (a buffer of one set is shorter than its tensor)");
         return -4;
     }
@@ -679,7 +718,10 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
     AmpDeviceState *host_mirror;
     AmpBiasTable bias;
     if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
-    const unsigned int stamp = amp_next_stamp(amp);
+    const unsigned long long stamp = amp_next_stamp(amp);
+    AmpDeviceState *pre, *post;
+    amp_take_records(amp, pre, post);
+    unsigned long long *overflow = &amp->d_block->overflow;
 
     hipStream_t st = l.ctx->stream;
     if (plan_a->num_chunks > 0) {
@@ -692,7 +734,7 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
         int count;
         if (!launch_geometry(*plan_a, vec, block, seg, count)) return -6;
 #define GM_LAUNCH_FUSED(V, N, B) \
-        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(amp->d_state, g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, bias, stamp)
+        amp_adam_fused_kernel<V, N, B><<<g.grid, B, 0, st>>>(pre, g.chunks, plan_b->d_chunks + (g.chunks - plan_a->d_chunks), g.shift, p, bias, stamp, overflow)
 #define GM_LAUNCH_FUSED_B(B)                                                              \
         if (vec == 4) { if (nt) GM_LAUNCH_FUSED(4, true, B); else GM_LAUNCH_FUSED(4, false, B); }        \
         else if (vec == 2) { if (nt) GM_LAUNCH_FUSED(2, true, B); else GM_LAUNCH_FUSED(2, false, B); }   \
@@ -707,7 +749,7 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
     // without an fp16 copy there is nothing to repair: one workgroup, for the epilogue alone
     const bool repair = plan_a->num_chunks > 0 && weight16_buffers;
     const unsigned int grid = !repair ? 1u : (plan_a->num_chunks < kRepairGrid ? plan_a->num_chunks : kRepairGrid);
-    amp_finalize_repair_kernel<<<grid, kBlock, 0, st>>>(amp->d_state, host_mirror, stamp, plan_a->d_chunks,
+    amp_finalize_repair_kernel<<<grid, kBlock, 0, st>>>(pre, post, host_mirror, overflow, stamp, plan_a->d_chunks,
                                                        plan_b->d_chunks, repair ? plan_a->num_chunks : 0u);
     return hip_ok(hipGetLastError(), "mixed-precision kernel launch") ? 0 : -6;
 }
@@ -779,6 +821,21 @@ try {
     std::lock_guard<std::mutex> lk(s->ctx->mu);
     if (!amp_download(s)) return -6;
     return s->h_pinned->current_set;
+} catch (...) {
+    note_exception();
+    return -6;
+}
+
+int gm_amp_state_set_current_set(uintptr_t amp_state, int current_set)
+try {
+    AmpState *s = amp_from_handle(amp_state);
+    if (!s) return -16;
+    if (current_set != 0 && current_set != 1) return -5;
+    if (!make_current(s->ctx)) return -6;
+    std::lock_guard<std::mutex> lk(s->ctx->mu);
+    if (!amp_download(s)) return -6;
+    s->h_pinned->current_set = current_set;
+    return amp_upload(s) ? 0 : -6;
 } catch (...) {
     note_exception();
     return -6;

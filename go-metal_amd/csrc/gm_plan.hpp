@@ -36,6 +36,7 @@ struct MultiTensorPlan {
     PlanSegment segment[2];
     int num_segments = 0;
     uint64_t total_elements = 0;
+    uint64_t kept_signature = 0;  // PlanLayout::kept_signature
 };
 
 // Returns the cached plan for this request or builds one (under ctx->mu, which

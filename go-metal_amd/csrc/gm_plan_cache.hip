@@ -139,6 +139,7 @@ static std::unique_ptr<MultiTensorPlan> build_plan(Context *ctx, const PlanReque
     plan->segment[1] = layout.segment[1];
     plan->num_segments = layout.num_segments;
     plan->total_elements = layout.total_elements;
+    plan->kept_signature = layout.kept_signature;
     const size_t count = layout.chunks.size();
     if (plan->status != 0 || count == 0) return plan;
     if (count > 0x7FFFFFFFull) {

@@ -120,6 +120,7 @@ void layout_plan(const PlanRequest &r, int requested_chunk, BufferLengthFn lengt
             break;
         }
         if (t.skip) continue;
+        out.kept_signature = (out.kept_signature ^ (uint64_t)(i + 1)) * 0x100000001B3ull;     // FNV-1a over indices
         const bool in_small_segment = small_chunk != 0 && t.numel < small_limit;
         const size_t step = (size_t)(in_small_segment ? small_chunk : chunk);
         std::vector<Chunk> &table = in_small_segment ? small_chunks : out.chunks;

@@ -121,6 +121,8 @@ struct PlanLayout {
     PlanSegment segment[2];
     int num_segments = 0;
     uint64_t total_elements = 0;
+    uint64_t kept_signature = 0;    // hash over the indices of the tensors that take part, in order: two
+                                    // layouts of the same sizes pair chunk for chunk only if it is equal
     std::vector<Chunk> chunks;      // segment 0's, then segment 1's
 };
 

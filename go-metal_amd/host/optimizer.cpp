@@ -439,10 +439,19 @@ Error AdamOptimizerState::EnableMixedPrecision(float initialScale, float growthF
     if (device == nullptr) return Errorf("device cannot be nil");
     if (!(initialScale > 0)) return Errorf("initial loss scale must be positive, got %f", initialScale);
     if (growthInterval <= 0) return Errorf("growth interval must be positive, got %d", growthInterval);
-    if (ampState) gm_amp_state_destroy(reinterpret_cast<uintptr_t>(ampState));
+    if (ampState) {
+        // a second call replaces the loss-scale state; steps still in flight finish first, and with ping-pong
+        // state on, the new device state is told which set is current (a fresh one would say set A)
+        if (ampPending > 0)
+            if (Error e = SyncAMP(); !e.empty()) return e;
+        gm_amp_state_destroy(reinterpret_cast<uintptr_t>(ampState));
+    }
     ampState = reinterpret_cast<Pointer>(gm_amp_state_create(reinterpret_cast<uintptr_t>(device), initialScale,
                                                              growthFactor, backoffFactor, growthInterval));
     if (ampState == nullptr) return Errorf("failed to create loss-scale state: %s", gm_last_error());
+    if (pingPong && currentSet != 0 &&
+        gm_amp_state_set_current_set(reinterpret_cast<uintptr_t>(ampState), currentSet) != 0)
+        return Errorf("failed to carry the current ping-pong set over: %s", gm_last_error());
     LossScale = initialScale;
     GrowthTracker = 0;
     ampPending = 0;

@@ -341,6 +341,10 @@ int execute_adam_amp_step_fused_async(uintptr_t device, uintptr_t *weight_a, uin
 /* 0 when set A holds the current weights and moments of the ping-pong step, 1 when set B does.
  * Waits for every step in flight.  -16: nil state; -6: HIP error. */
 int gm_amp_state_current_set(uintptr_t amp_state);
+/* Tells a loss-scale state which set holds the current weights and moments (0: A, 1: B): for a state
+ * created anew over ping-pong buffers that are already in use.  Waits for every step in flight.
+ * -16: nil state; -5: not 0 or 1; -6: HIP error.  No counterpart in the reference. */
+int gm_amp_state_set_current_set(uintptr_t amp_state, int current_set);
 
 /* allocate_metal_buffer with a say in where the buffer starts: the handle's address is congruent to
  * phase_bytes modulo 2 MiB (phase_bytes: a multiple of 256 below 2 MiB).  No counterpart in the
@@ -361,7 +365,10 @@ uintptr_t gm_allocate_buffer_phased(uintptr_t device, int size, int device_type,
  * device.  Limits: 4096 tensors and 32768 chunk descriptors (about 2.1e9 parameters in chunks of
  * 65536 elements); beyond them -17 and a message in gm_last_error, nothing launched.  Every call on
  * a GPU rewrites that GPU's one table: calls are ordered on the library's stream, and calls that
- * overlap on one GPU by any other means race.
+ * overlap on one GPU by any other means race.  Under graph capture the call's scalars (learning rate, the
+ * bias corrections of step_count) and the handle records travel as kernel arguments and are frozen
+ * into the captured nodes: a replay repeats THAT step's corrections, so capture per step count or set
+ * the nodes' kernel parameters before each replay (no test here exercises capture).
  * -1 device 0; -3 no GPU; -4 a required handle is 0 (nothing updated); -6 HIP error; -17 over the limits. */
 int execute_adam_step_noalloc(uintptr_t device, uintptr_t *weight_buffers, uintptr_t *gradient_buffers,
                               uintptr_t *momentum_buffers, uintptr_t *variance_buffers, int num_weights,

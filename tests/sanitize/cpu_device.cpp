@@ -498,6 +498,13 @@ int execute_adam_amp_step_async(uintptr_t device, uintptr_t *w, uintptr_t *g16, 
 }
 
 int gm_amp_state_current_set(uintptr_t h) { return h ? reinterpret_cast<AmpState *>(h)->current_set : -16; }
+int gm_amp_state_set_current_set(uintptr_t h, int set)
+{
+    if (!h) return -16;
+    if (set != 0 && set != 1) return -5;
+    reinterpret_cast<AmpState *>(h)->current_set = set;
+    return 0;
+}
 
 // The one-pass step over ping-pong state: the current set is read, the other one written.
 int execute_adam_amp_step_fused(uintptr_t device, uintptr_t *wa, uintptr_t *ma, uintptr_t *va, uintptr_t *wb,

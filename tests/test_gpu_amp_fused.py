@@ -238,6 +238,50 @@ def test_fused_step_argument_errors(dev):
             dev.free(h)
 
 
+def test_fused_step_refuses_sets_whose_skipped_tensors_differ(dev):
+    """Two tensors of one size, the first one's weight buffer too short in set A only and the second one's in set B
+    only: each set skips one tensor, so chunk counts, chunk sizes and element totals of the two layouts agree, and
+    pairing them chunk for chunk would read one tensor and write the other.  The step is refused (-4) and nothing is
+    written."""
+    lib, D = dev.lib, dev.handle
+    n = 5000
+    arr = pkg.handle_array
+    full = {k: [dev.from_numpy(np.full(n, 1.5 + i, np.float32)) for i in range(2)] for k in ("wa", "ma", "va", "wb", "mb", "vb")}
+    short = [dev.from_numpy(np.full(n - 16, 9.0, np.float32)) for _ in range(2)]
+    g16 = [dev.alloc(2 * n, zero=True) for _ in range(2)]
+    w16 = [dev.from_numpy(np.full(n, 0x3C00, np.uint16)) for _ in range(2)]
+    bs = pkg.int_array([4 * n, 4 * n])
+    amp = lib.gm_amp_state_create(D, 65536.0, 2.0, 0.5, 2000)
+    sk = ctypes.c_int(-1)
+    try:
+        wa = [short[0], full["wa"][1]]
+        wb = [full["wb"][0], short[1]]
+        rc = lib.execute_adam_amp_step_fused(D, arr(wa), arr(full["ma"]), arr(full["va"]), arr(wb), arr(full["mb"]),
+                                             arr(full["vb"]), arr(g16), arr(w16), 2, bs, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1,
+                                             amp, ctypes.byref(sk), None, None, None)
+        assert rc == -4 and b"same tensors" in lib.gm_last_error(), (rc, lib.gm_last_error())
+        assert lib.gm_amp_state_current_set(amp) == 0
+        for k, hs in full.items():
+            for i, h in enumerate(hs):
+                assert np.all(dev.to_numpy(h, n) == np.float32(1.5 + i)), (k, i)
+        for h in w16:
+            assert np.all(dev.to_numpy(h, n, np.uint16) == 0x3C00)
+        # the same tensor short in both sets is skipped in both: allowed, and the other tensor is stepped
+        wb2 = [short[1], full["wb"][1]]
+        rc = lib.execute_adam_amp_step_fused(D, arr(wa), arr(full["ma"]), arr(full["va"]), arr(wb2), arr(full["mb"]),
+                                             arr(full["vb"]), arr(g16), arr(w16), 2, bs, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1,
+                                             amp, ctypes.byref(sk), None, None, None)
+        assert rc == 0 and sk.value == 0, (rc, lib.gm_last_error())
+        assert np.all(dev.to_numpy(full["wb"][0], n) == np.float32(1.5))          # tensor 0: skipped, untouched
+        assert np.all(dev.to_numpy(full["mb"][0], n) == np.float32(1.5))
+        assert not np.all(dev.to_numpy(full["mb"][1], n) == np.float32(2.5))      # tensor 1: set B written
+    finally:
+        lib.gm_amp_state_destroy(amp)
+        for hs in list(full.values()) + [short, g16, w16]:
+            for h in hs:
+                dev.free(h)
+
+
 def test_in_place_and_one_pass_steps_share_one_loss_scale_state(dev):
     """Both forms advance the same device state and tell an overflow by the same per-step stamp: alternated on one
     list (the in-place step working on whichever set is current), with dropped steps next to each other, before

@@ -291,6 +291,58 @@ def test_step_amp_async_through_the_mirror(env):
         dev.free(h)
 
 
+def test_enabling_mixed_precision_again_keeps_the_current_ping_pong_set(env):
+    """EnableMixedPrecision called a second time (another initial scale, say) replaces the loss-scale state on the
+    device.  After an odd number of applied ping-pong steps the shadow set is the current one: the new state must
+    be told, or the next step would read the stale set A and overwrite the real weights in B."""
+    dev, mm = env
+    rng = np.random.default_rng(23)
+    sizes = [int(np.prod(s)) for s in SHAPES]
+    cfg, hyper = CASES[2][1], CASES[2][2]
+    for applied_before in (1, 2):
+        opt = make(env, "adam", cfg)
+        w = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+        dw = [dev.from_numpy(a) for a in w]
+        w16 = [a.astype(np.float16).view(np.uint16) for a in w]
+        dw16 = [dev.from_numpy(h) for h in w16]
+        dg = [dev.alloc(2 * n + 2) for n in sizes]
+        m = [np.zeros(n, np.float32) for n in sizes]
+        v = [np.zeros(n, np.float32) for n in sizes]
+        assert opt.SetWeightBuffers(dw) is None
+        assert opt.EnableMixedPrecision(4096.0, 2.0, 0.5, 100) is None and opt.EnablePingPong() is None
+        st = oracle().amp_state(4096.0, 2.0, 0.5, 100)
+
+        def step(use_async):
+            g16 = [(rng.normal(0, 1e-4, n) * st.scale).astype(np.float16).view(np.uint16) for n in sizes]
+            for h, g in zip(dg, g16):
+                dev.upload(h, g)
+            if use_async:
+                assert opt.StepAMPAsync(dg, dw16) is None
+            else:
+                assert opt.StepAMP(dg, dw16) == (False, None)
+            assert oracle().adam_amp(w, g16, m, v, w16, state=st, **hyper) == 0
+
+        for k in range(applied_before):
+            step(use_async=(k == applied_before - 1))          # the last one still in flight when the state is replaced
+        # a new loss-scale state with another scale; the oracle's state is replaced the same way
+        assert opt.EnableMixedPrecision(1024.0, 2.0, 0.5, 7) is None
+        assert opt.current_set() == applied_before % 2 and opt.GetStepCount() == applied_before
+        st2 = oracle().amp_state(1024.0, 2.0, 0.5, 7)
+        st2.step_count = st.step_count
+        st = st2
+        for k in range(3):
+            step(use_async=False)
+        assert opt.current_set() == (applied_before + 3) % 2 and opt.GetStepCount() == applied_before + 3
+        for k, n in enumerate(sizes):
+            for name, host in (("weight", w), ("momentum", m), ("variance", v)):
+                assert np.array_equal(dev.to_numpy(opt.state_buffer(name, k), n).view(np.uint32), host[k].view(np.uint32)), (applied_before, name, k)
+            assert np.array_equal(dev.to_numpy(dw16[k], n, np.uint16), w16[k]), (applied_before, k)
+        opt.Cleanup()
+        opt.free()
+        for h in dw + dw16 + dg:
+            dev.free(h)
+
+
 def test_ping_pong_mixed_precision_through_the_mirror(env):
     """EnablePingPong: StepAMP / StepAMPAsync run the one-pass step over two sets of weights and moments.  The
     current weights (state_buffer "weight"), the moments GetState reads, the fp16 copy and every counter follow
