@@ -1,0 +1,130 @@
+"""The Go sources under integration/go (the files a go-metal maintainer copies over a checkout) against the C
+header they bind: no Go toolchain exists here, so they cannot be compiled; what can be checked mechanically is
+that every C function they call is declared in include/gometal_hip.h with the number of arguments they pass, and
+that every error string and hook they rely on is the one the tested C++ mirror uses."""
+import glob
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GO = os.path.join(ROOT, "integration", "go")
+C_TYPES = {"int", "float", "uintptr_t", "double", "char", "size_t", "uint64_t"}
+
+
+def split_top_level(args):
+    """Arguments of a call or a prototype, split at commas outside parentheses and brackets."""
+    parts, depth, cur = [], 0, ""
+    for ch in args:
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+        if ch == "," and depth == 0:
+            parts.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        parts.append(cur.strip())
+    return parts
+
+
+def header_prototypes():
+    text = open(os.path.join(ROOT, "include", "gometal_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    protos = {}
+    for m in re.finditer(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(([^()]*)\)\s*;", text):
+        name, args = m.group(1), m.group(2).strip()
+        protos[name] = 0 if args in ("", "void") else len(split_top_level(args))
+    return protos
+
+
+def go_c_calls(path):
+    """(name, number of arguments, line) of every C.name(...) call in a Go file, casts to C types left out."""
+    text = open(path).read()
+    text = re.sub(r"/\*.*?\*/", lambda m: "\n" * m.group(0).count("\n"), text, flags=re.S)    # the cgo preamble
+    text = re.sub(r"//[^\n]*", "", text)
+    calls = []
+    for m in re.finditer(r"\bC\.([A-Za-z_][A-Za-z0-9_]*)\s*\(", text):
+        name = m.group(1)
+        if name in C_TYPES:
+            continue
+        depth, i = 1, m.end()
+        while depth:
+            depth += {"(": 1, ")": -1}.get(text[i], 0)
+            i += 1
+        calls.append((name, len(split_top_level(text[m.end():i - 1])), text.count("\n", 0, m.start()) + 1))
+    return calls
+
+
+def go_files():
+    files = sorted(glob.glob(os.path.join(GO, "**", "*.go"), recursive=True))
+    assert len(files) >= 5
+    return files
+
+
+def test_every_c_function_the_go_wrappers_call_is_declared_with_that_arity():
+    protos = header_prototypes()
+    assert protos["execute_adam_amp_step"] == 18 and protos["execute_adam_amp_step_fused"] == 22
+    assert protos["gm_allocate_buffer_phased"] == 4 and protos["gm_amp_state_query"] == 5
+    seen = set()
+    for path in go_files():
+        for name, nargs, line in go_c_calls(path):
+            where = f"{os.path.relpath(path, ROOT)}:{line}"
+            assert name in protos, f"{where}: C.{name} is not declared in include/gometal_hip.h"
+            assert nargs == protos[name], f"{where}: C.{name} called with {nargs} arguments, declared with {protos[name]}"
+            seen.add(name)
+    assert {"execute_adam_amp_step", "execute_adam_amp_step_async", "execute_adam_amp_step_fused",
+            "execute_adam_amp_step_fused_async", "gm_allocate_buffer_phased", "gm_amp_state_create",
+            "gm_amp_state_destroy", "gm_amp_state_query", "gm_amp_state_set", "gm_amp_state_set_step_count",
+            "gm_amp_state_current_set", "gm_amp_state_set_current_set", "gm_synchronize"} <= seen
+
+
+def test_go_files_are_plausible_go():
+    """Balanced braces and parentheses, a package clause, the build tag on the files that need the library."""
+    for path in go_files():
+        text = open(path).read()
+        code = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        code = re.sub(r"//[^\n]*", "", code)
+        code = re.sub(r'"(\\.|[^"\\])*"', '""', code)
+        for a, b in ("()", "{}", "[]"):
+            assert code.count(a) == code.count(b), (path, a)
+        package = os.path.basename(os.path.dirname(path))
+        assert re.search(rf"^package {package}$", text, flags=re.M), path
+        if "C." in code or "cgo_bridge.AMPSet" in code or "AllocateMetalBufferPhased" in code:
+            assert text.startswith("//go:build linux && amd64\n"), path
+
+
+def test_go_error_strings_are_the_mirrors():
+    """The Go methods were written from the C++ mirror the GPU tests drive (host/optimizer.cpp, host/bridge.cpp):
+    every error string of theirs must occur there too (format verbs aside: %v in Go where C++ has %s)."""
+    mirror = "".join(open(os.path.join(ROOT, "go-metal_amd", "host", f)).read()
+                     for f in ("optimizer.cpp", "bridge.cpp", "memory_manager.cpp"))
+    mirror = mirror.replace('"\n', '"').replace("%s", "%v")
+    mirror = re.sub(r'"\s*\n\s*"', "", mirror)
+    own = {"loss-scale state query failed with error code: %d", "loss-scale state update failed with error code: %d",
+           "loss-scale state step count update failed with error code: %d", "failed to create loss-scale state",
+           "device synchronisation failed with error code: %d",
+           "failed to allocate Metal buffer of size %d at phase %d"}          # the wrappers' own, one per new C call
+    for name in ("optimizer/adam_amp.go", "cgo_bridge/bridge_amp_linux.go"):
+        text = open(os.path.join(GO, name)).read()
+        for m in re.finditer(r'fmt\.Errorf\("((?:\\.|[^"\\])*)"', text):
+            msg = m.group(1)
+            assert msg in own or msg in mirror, (name, msg)
+
+
+def test_hooks_named_in_the_go_files_exist():
+    """adam_amp.go tells the maintainer which lines of adam.go call into it; those functions are defined."""
+    text = open(os.path.join(GO, "optimizer", "adam_amp.go")).read()
+    for fn in ("beforeStep", "cleanupAMP", "CurrentWeightBuffers", "CurrentMomentumBuffers", "CurrentVarianceBuffers",
+               "finishPendingAMP", "EnableMixedPrecision", "EnablePingPong", "StepAMP", "StepAMPAsync", "SyncAMP"):
+        assert re.search(rf"^func \(adam \*AdamOptimizerState\) {fn}\(", text, flags=re.M), fn
+    mem = open(os.path.join(GO, "memory", "manager_state.go")).read()
+    for fn in ("AllocateStateBuffer", "AllocateBufferAtPhase", "releasePlaced"):
+        assert re.search(rf"^func \(mm \*MemoryManager\) {fn}\(", mem, flags=re.M), fn
+    # the constants are the C++ mirror's
+    hpp = open(os.path.join(ROOT, "go-metal_amd", "host", "memory_manager.hpp")).read()
+    assert "kStatePhases[3] = {512 << 10, 1536 << 10, 1 << 20}" in hpp and "[3]int{512 << 10, 1536 << 10, 1 << 20}" in mem
+    assert "kShadowWeightPhase = 1 << 20" in hpp and "ShadowWeightPhase = 1 << 20" in mem
+    assert "kPhasedMinBytes = 16 << 20" in hpp and "PhasedMinBytes = 16 << 20" in mem

@@ -5,6 +5,9 @@ scale regenerated on the device for every step, +inf / -inf / NaN written into o
 seeded 0.5 % of steps, loss scale 65536 with backoff x0.5 and growth x2 every 2000 clean steps.
 config 5 (mixed-precision variant): 1,012,301,824 parameters in 400 tensors, weight decay 1e-4, 20 steps.
 
+A third schedule (growth every 100 clean steps, an injection on about 1 % of 1000 steps) makes the scale move up
+and down at full size with gradients that never underflow.
+
 Every step's (skipped, scale, clean-step counter, step count) must equal the CPU oracle's, and weights,
 moments and the fp16 weight copy are compared bit for bit at checkpoints (every 500 steps / steps 1, 10, 20).
 The oracle consumes the very gradients the device generated (read back once per step) and runs in a worker
@@ -35,8 +38,9 @@ def dev():
     return d
 
 
-def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed, fused=False):
-    """inject_at: {step index: (tensor, element, fp16 bits)}; checkpoints: step indices (0-based) after which
+def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed, fused=False,
+                 loss_scale=(65536.0, 2.0, 0.5, 2000)):
+    """loss_scale: (initial scale, growth factor, backoff factor, growth interval).  inject_at: {step index: (tensor, element, fp16 bits)}; checkpoints: step indices (0-based) after which
     all buffers are compared.  fused: the one-pass ping-pong step (two sets of weights and moments on the device,
     the fp16 copy kept as half of the current weights from the start) instead of the in-place step."""
     pkg, lib, D, o = load_package(), dev.lib, dev.handle, oracle()
@@ -63,7 +67,7 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed, f
     c_g16 = arr([d_g16 + 2 * int(off) for off in offsets[:-1]])
     c_w16 = arr([d_w16 + 2 * int(off) for off in offsets[:-1]])
     bs = pkg.int_array([4 * s for s in sizes])
-    amp = lib.gm_amp_state_create(D, 65536.0, 2.0, 0.5, 2000)
+    amp = lib.gm_amp_state_create(D, *loss_scale)
     assert amp
 
     # ---- oracle side
@@ -71,7 +75,7 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed, f
     v_host = [np.zeros(s, np.float32) for s in sizes]
     w16_host = [a.astype(np.float16).view(np.uint16) if fused else np.zeros(s, np.uint16)
                 for a, s in zip(w_host, sizes)]
-    st = o.amp_state(65536.0, 2.0, 0.5, 2000)
+    st = o.amp_state(*loss_scale)
     g_buffers = [np.empty((2 * total + 3) // 4, np.uint32) for _ in range(2)]
     free_buffers, work = queue.Queue(), queue.Queue(maxsize=1)
     for b in range(2):
@@ -116,7 +120,7 @@ def run_schedule(dev, name, sizes, hyper, steps, inject_at, checkpoints, seed, f
             assert np.array_equal(got16[offsets[k]:offsets[k + 1]], w16_host[k]), (context, "w16", k)
 
     gpu_trace = []
-    scale, applied = 65536.0, 0
+    scale, applied = loss_scale[0], 0
     t0 = time.time()
     try:
         for k in range(steps):
@@ -178,10 +182,56 @@ def test_config4_full_size_5000_steps(dev):
         inject[int(k)] = (t, int(rng.integers(0, sizes[t])), [0x7C00, 0xFC00, 0x7E00][j % 3])
     assert len(inject) > 10
     trace = run_schedule(dev, "config 4", sizes, hyper, 5000, inject, {499 + 500 * i for i in range(10)}, seed=4)
-    # the schedule really exercised both directions of the scale
-    scales = {t[1] for t in trace}
-    assert len(scales) >= 4 and min(scales) < 65536.0
+    # In this schedule the scale only ever drops: a growth needs 2000 clean steps in a row, and with an injection
+    # on 0.5 % of steps that happens with probability 4e-5.  The scale ends at 65536 / 2^len(inject), and from
+    # about step 3500 on half(N(0, 1e-4) x scale) underflows to zero.  Growth, and gradients that stay alive to the
+    # end, are what test_full_size_growth_and_backoff below is for.
+    scales = [t[1] for t in trace]
+    assert all(b <= a for a, b in zip(scales, scales[1:])) and scales[-1] == 65536.0 / 2.0 ** len(inject)
     assert trace[-1][3] == 5000 - len(inject)
+
+
+def growth_schedule(steps, sizes, seed, rate=0.01):
+    """Injections on a seeded `rate` of the steps, and the loss-scale trajectory they produce from 65536 with growth
+    x2 every 100 clean steps and backoff x0.5, computed here by a plain state machine: (inject, scales, growths,
+    backoffs)."""
+    rng = np.random.default_rng(seed)
+    chosen = np.flatnonzero(rng.random(steps) < rate)
+    inject = {}
+    for j, k in enumerate(chosen):
+        t = int(rng.integers(0, len(sizes)))
+        inject[int(k)] = (t, int(rng.integers(0, sizes[t])), [0x7C00, 0xFC00, 0x7E00][j % 3])
+    scale, tracker, scales, growths, backoffs = 65536.0, 0, [], 0, 0
+    for k in range(steps):
+        if k in inject:
+            scale, tracker, backoffs = scale * 0.5, 0, backoffs + 1
+        else:
+            tracker += 1
+            if tracker == 100:
+                scale, tracker, growths = scale * 2.0, 0, growths + 1
+        scales.append(scale)
+    return inject, scales, growths, backoffs
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["in_place", "one_pass"])
+def test_full_size_growth_and_backoff(dev, fused):
+    """125,000,000 parameters in 60 tensors, 1000 steps, growth every 100 clean steps, an inf / NaN on about 1 % of
+    steps: the scale goes up and down several times and stays between 2^10 and 2^20, so the fp16 gradients
+    N(0, 1e-4) x scale never underflow and every applied step is a real update to the end of the run.  Every
+    step's (skipped, scale, clean-step counter, step count) and, at three checkpoints, every buffer equal the
+    oracle's, for the in-place step and for the one-pass step over ping-pong state."""
+    sizes = amp_125m_sizes()
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)
+    inject, scales, growths, backoffs = growth_schedule(1000, sizes, seed=0x6D657461 + 45)
+    assert growths >= 3 and backoffs >= 3 and 2.0 ** 10 <= min(scales) and max(scales) <= 2.0 ** 20, (growths, backoffs, min(scales), max(scales))
+    trace = run_schedule(dev, "growth and backoff, " + ("one pass" if fused else "in place"), sizes, hyper, 1000, inject,
+                         {332, 665, 999}, seed=44, fused=fused, loss_scale=(65536.0, 2.0, 0.5, 100))
+    got = [t[1] for t in trace]
+    assert got == scales
+    ups = sum(1 for a, b in zip(got, got[1:]) if b > a)
+    downs = sum(1 for a, b in zip(got, got[1:]) if b < a)
+    assert ups >= 3 and downs >= 3 and min(got) >= 2.0 ** 10 and max(got) <= 2.0 ** 20
+    assert trace[-1][3] == 1000 - len(inject)
 
 
 def test_config5_mixed_precision_full_size_20_steps(dev):
@@ -192,19 +242,20 @@ def test_config5_mixed_precision_full_size_20_steps(dev):
     assert [t[0] for t in trace].count(1) == 2 and trace[-1][1] == 16384.0 and trace[-1][3] == 18
 
 
-def test_config4_full_size_one_pass_step_1500_steps(dev):
-    """The first 1500 steps of the same schedule through the one-pass ping-pong step."""
+def test_config4_full_size_one_pass_step_5000_steps(dev):
+    """The same 5000-step schedule through the one-pass ping-pong step."""
     sizes = amp_125m_sizes()
     hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0)
     rng = np.random.default_rng(0x6D657461 + 4)
-    chosen = [int(k) for k in np.flatnonzero(rng.random(5000) < 0.005) if k < 1500]
+    chosen = np.flatnonzero(rng.random(5000) < 0.005)
     inject = {}
     for j, k in enumerate(chosen):
         t = int(rng.integers(0, len(sizes)))
-        inject[k] = (t, int(rng.integers(0, sizes[t])), [0x7C00, 0xFC00, 0x7E00][j % 3])
-    assert len(inject) >= 5
-    trace = run_schedule(dev, "config 4, one pass", sizes, hyper, 1500, inject, {499, 999, 1499}, seed=4, fused=True)
-    assert trace[-1][3] == 1500 - len(inject)
+        inject[int(k)] = (t, int(rng.integers(0, sizes[t])), [0x7C00, 0xFC00, 0x7E00][j % 3])
+    assert len(inject) > 10
+    trace = run_schedule(dev, "config 4, one pass", sizes, hyper, 5000, inject, {499 + 500 * i for i in range(10)}, seed=4,
+                         fused=True)
+    assert trace[-1][3] == 5000 - len(inject) and trace[-1][1] == 65536.0 / 2.0 ** len(inject)
 
 
 def test_config5_mixed_precision_full_size_one_pass_step_20_steps(dev):
