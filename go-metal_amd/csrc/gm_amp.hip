@@ -26,12 +26,16 @@
 
 #include "../../include/gometal_hip.h"
 
+#include <chrono>
+#include <cstddef>
 #include <cstring>
+#include <thread>
 
 namespace gm {
 
 constexpr float kMinLossScale = 1.17549435e-38f;   // FLT_MIN
 constexpr float kMaxLossScale = 3.40282347e+38f;   // FLT_MAX
+constexpr int kAmpSpinMicroseconds = 100;   // how long the host spins on a pinned stamp before it naps or blocks
 constexpr int kCheckUnroll = 4;           // 16-byte loads in flight per lane in the overflow check
 
 // Loss-scale state machine, resident in HBM next to the tensors.
@@ -39,7 +43,7 @@ struct alignas(16) AmpDeviceState {
     // head: the 16 bytes every workgroup of the update kernel reads with one scalar load
     int current_set;        // ping-pong step: 0 = set A holds the current weights and moments, 1 = set B
     float inv_scale;        // 1.0f / scale, kept by whoever changes scale (IEEE division on host and device alike)
-    int unused;
+    int skipped_steps;      // steps dropped so far
     int applied_steps;      // steps applied so far (the optimizer's StepCount): +1 per clean step
     // tail
     float scale;
@@ -48,9 +52,11 @@ struct alignas(16) AmpDeviceState {
     float growth_factor;
     float backoff_factor;
     int growth_interval;
-    int skipped_steps;      // steps dropped so far
-    int pad;
+    unsigned long long stamp;   // the stamp of the step this record is the post-state of (0: set by the host).  In
+                                // the pinned host copy it is written last: the host knows the record is complete
+                                // when it reads the stamp it expects
 };
+static_assert(offsetof(AmpDeviceState, stamp) == 40, "AmpDeviceState layout");
 static_assert(sizeof(AmpDeviceState) == 48, "AmpDeviceState layout");
 
 // What a loss-scale state keeps on the device: the record the next step reads and the record it
@@ -127,7 +133,7 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, unsigned long long *
 // writes its post-state into the record the next step reads.  found: this step's gradients held
 // an inf / NaN.
 __device__ inline void amp_advance(const AmpDeviceState *pre, AmpDeviceState *post, AmpDeviceState *host_mirror,
-                                   bool found, int ping_pong)
+                                   bool found, int ping_pong, unsigned long long stamp)
 {
     AmpDeviceState st = *pre;
     // The scale stays a normal, finite fp32 number whatever the run does: a growth that would
@@ -151,10 +157,19 @@ __device__ inline void amp_advance(const AmpDeviceState *pre, AmpDeviceState *po
     }
     st.inv_scale = 1.0f / st.scale;
     st.last_skipped = found ? 1 : 0;
+    st.stamp = stamp;
     *post = st;
-    // The post-state also goes straight into pinned host memory: the host reads it once the
-    // stream (or the event recorded after this launch) has completed, without a copy launch.
-    if (host_mirror) *host_mirror = st;
+    // The post-state also goes straight into pinned host memory, its stamp last and behind a
+    // system-scope fence: the host reads the record without a copy launch, either after the stream
+    // has completed or as soon as it sees the stamp of the step it is waiting for.
+    if (host_mirror) {
+        const unsigned long long *src = reinterpret_cast<const unsigned long long *>(&st);
+        unsigned long long *dst = reinterpret_cast<unsigned long long *>(host_mirror);
+#pragma unroll
+        for (int k = 0; k < 5; k++) dst[k] = src[k];
+        __threadfence_system();
+        __hip_atomic_store(&host_mirror->stamp, stamp, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 // The bias corrections of the step count the device has reached: entry (applied - base) of the
@@ -187,7 +202,7 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
     const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
     const bool found = seen == stamp;
-    if (post != nullptr && blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 0);
+    if (post != nullptr && blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 0, stamp);
     // (the weight pointer is never null; testing it here makes the compiler fetch the whole
     // descriptor before the branch instead of the count first and the addresses after it)
     if (found | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
@@ -307,7 +322,7 @@ __global__ void amp_finalize_kernel(const AmpDeviceState *pre, AmpDeviceState *p
                                     const unsigned long long *overflow, unsigned long long stamp, int ping_pong)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    amp_advance(pre, post, host_mirror, *overflow == stamp, ping_pong);
+    amp_advance(pre, post, host_mirror, *overflow == stamp, ping_pong, stamp);
 }
 
 // Epilogue of the ping-pong step, and the repair of the fp16 weight copy, in one launch.  After a
@@ -323,7 +338,7 @@ amp_finalize_repair_kernel(const AmpDeviceState *pre, AmpDeviceState *post, AmpD
                            const Chunk *__restrict__ set_a, const Chunk *__restrict__ set_b, uint32_t num_chunks)
 {
     const bool found = *overflow == stamp;
-    if (blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 1);
+    if (blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 1, stamp);
     if (!found) return;
     const Chunk *current = pre->current_set != 0 ? set_b : set_a;      // a dropped step keeps the current set
     for (uint32_t c = blockIdx.x; c < num_chunks; c += gridDim.x) {
@@ -348,7 +363,7 @@ struct AmpState {
     AmpDeviceBlock *d_block;
     int slot;                            // which record of d_block the next step reads (the state as of now)
     AmpDeviceState *h_pinned;            // kAmpMaxInFlight + 1 slots: [0] synchronous read-backs, [1..] the ring
-    hipEvent_t ring_event[kAmpMaxInFlight];
+    unsigned long long ring_stamp[kAmpMaxInFlight];    // stamp of the asynchronous step whose post-state a ring slot awaits
     // asynchronous steps: issue numbers count execute_adam_amp_step_async calls
     uint64_t issued;                     // steps issued so far
     uint64_t confirmed_issue;            // newest step whose post-state the host has seen
@@ -384,27 +399,74 @@ static bool amp_download(AmpState *s)
     return true;
 }
 
-// Takes note of the asynchronous steps that have finished since the last look.  With
-// must_free_slot, blocks until at most kAmpMaxInFlight - 2 steps are unconfirmed, so that the
-// next step's bias table and ring slot are available.
+// Whether the post-state of asynchronous step `issue` has arrived in its ring slot.
+static bool amp_arrived(const AmpState *s, uint64_t issue)
+{
+    const int slot = (int)(issue % kAmpMaxInFlight);
+    return __atomic_load_n(&s->h_pinned[1 + slot].stamp, __ATOMIC_ACQUIRE) == s->ring_stamp[slot];
+}
+
+// Takes note of the asynchronous steps that have finished since the last look: a step has
+// finished when its ring slot holds its stamp (the device writes the stamp last).  No HIP call
+// in the common case.  With must_free_slot, waits until at most kAmpMaxInFlight - 2 steps are
+// unconfirmed, so that the next step's bias table and ring slot are available: a short spin for
+// steps of microseconds, then naps while the stream is busy; a stream that has drained or
+// failed ends the wait, so it cannot outlast the work it waits for.
 static bool amp_poll(AmpState *s, bool must_free_slot)
 {
+    const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(kAmpSpinMicroseconds);
     for (;;) {
-        while (s->confirmed_issue < s->issued) {
-            const uint64_t next = s->confirmed_issue + 1;
-            const hipError_t q = hipEventQuery(s->ring_event[next % kAmpMaxInFlight]);
-            if (q == hipErrorNotReady) {
-                (void)hipGetLastError();     // "not ready" is an answer, not a failure to report later
-                break;
-            }
-            if (!hip_ok(q, "hipEventQuery")) return false;
-            s->confirmed_issue = next;
-            s->confirmed_applied = s->h_pinned[1 + next % kAmpMaxInFlight].applied_steps;
+        while (s->confirmed_issue < s->issued && amp_arrived(s, s->confirmed_issue + 1)) {
+            s->confirmed_issue += 1;
+            s->confirmed_applied = s->h_pinned[1 + s->confirmed_issue % kAmpMaxInFlight].applied_steps;
         }
         if (!must_free_slot || s->issued - s->confirmed_issue <= (uint64_t)kAmpMaxInFlight - 2) return true;
-        const uint64_t oldest = s->confirmed_issue + 1;
-        if (!hip_ok(hipEventSynchronize(s->ring_event[oldest % kAmpMaxInFlight]), "hipEventSynchronize"))
+        if (std::chrono::steady_clock::now() < spin_until) continue;
+        const hipError_t q = hipStreamQuery(s->ctx->stream);
+        if (q == hipErrorNotReady) {
+            (void)hipGetLastError();     // "not ready" is an answer, not a failure to report later
+            std::this_thread::sleep_for(std::chrono::microseconds(20));
+            continue;
+        }
+        if (!hip_ok(q, "hipStreamQuery")) return false;
+        // the stream is empty: every step has written its slot
+        if (!amp_arrived(s, s->issued)) {
+            set_error("a mixed-precision step finished without reporting its state");
             return false;
+        }
+    }
+}
+
+// Waits until the post-state of the synchronous step with this stamp has arrived in pinned slot 0
+// (the device writes the stamp last).  The in-place step reports from the first workgroup of its
+// update launch, as soon as the check has finished, so its outcome is known long before the
+// update has drained: the wait spins briefly, then naps while the stream is busy (naps: true).
+// The one-pass step reports from its last launch, when the stream is about to drain: after the
+// spin the stream's own wait is the cheaper one (naps: false).  A stream that has drained or
+// failed ends either wait.
+static bool amp_wait_outcome(AmpState *s, unsigned long long stamp, bool naps)
+{
+    const unsigned long long *word = &s->h_pinned->stamp;
+    const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(kAmpSpinMicroseconds);
+    while (std::chrono::steady_clock::now() < spin_until)
+        if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == stamp) return true;
+    for (;;) {
+        if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == stamp) return true;
+        if (!naps) {
+            if (!hip_ok(hipStreamSynchronize(s->ctx->stream), "hipStreamSynchronize")) return false;
+        } else {
+            const hipError_t q = hipStreamQuery(s->ctx->stream);
+            if (q == hipErrorNotReady) {
+                (void)hipGetLastError();
+                std::this_thread::sleep_for(std::chrono::microseconds(20));
+                continue;
+            }
+            if (!hip_ok(q, "hipStreamQuery")) return false;
+        }
+        // the stream is empty: the step has reported
+        if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == stamp) return true;
+        set_error("a mixed-precision step finished without reporting its state");
+        return false;
     }
 }
 
@@ -412,8 +474,6 @@ static void amp_free(AmpState *s)
 {
     if (s->d_block) (void)hipFree(s->d_block);
     if (s->h_pinned) (void)hipHostFree(s->h_pinned);
-    for (hipEvent_t e : s->ring_event)
-        if (e) (void)hipEventDestroy(e);
     s->magic = 0;
     delete s;
 }
@@ -442,8 +502,6 @@ try {
               hip_ok(hipMemsetAsync(s->d_block, 0, sizeof(AmpDeviceBlock), ctx->stream), "hipMemsetAsync(amp state)") &&
               hip_ok(hipHostMalloc(&s->h_pinned, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState),
                                    hipHostMallocDefault), "hipHostMalloc(amp state)");
-    for (int k = 0; ok && k < kAmpMaxInFlight; k++)
-        ok = hip_ok(hipEventCreateWithFlags(&s->ring_event[k], hipEventDisableTiming), "hipEventCreate");
     if (ok) {
         std::memset(s->h_pinned, 0, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState));
         s->h_pinned->scale = init_scale;
@@ -640,6 +698,7 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     AmpBiasTable bias;
     if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
     const unsigned long long stamp = amp_next_stamp(amp);
+    if (async) amp->ring_stamp[(amp->issued + 1) % kAmpMaxInFlight] = stamp;
     AmpDeviceState *pre, *post;
     amp_take_records(amp, pre, post);
     unsigned long long *overflow = &amp->d_block->overflow;
@@ -719,6 +778,7 @@ static int amp_enqueue_fused(uintptr_t device, AmpState *amp, uintptr_t *const s
     AmpBiasTable bias;
     if (!amp_bias_and_mirror(amp, async, beta1, beta2, step_count, bias, host_mirror)) return -6;
     const unsigned long long stamp = amp_next_stamp(amp);
+    if (async) amp->ring_stamp[(amp->issued + 1) % kAmpMaxInFlight] = stamp;
     AmpDeviceState *pre, *post;
     amp_take_records(amp, pre, post);
     unsigned long long *overflow = &amp->d_block->overflow;
@@ -771,7 +831,9 @@ try {
                              variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
                              beta1, beta2, epsilon, weight_decay, step_count, false, l, lock))
         return rc;
-    if (!hip_ok(hipStreamSynchronize(l.ctx->stream), "hipStreamSynchronize")) return -6;
+    // returns once the step's outcome is known; its update launch may still be running, and
+    // everything that reads its results is ordered behind it on the library's stream
+    if (!amp_wait_outcome(amp, amp->last_stamp, true)) return -6;
     amp->confirmed_issue = amp->issued;
     amp->confirmed_applied = amp->h_pinned->applied_steps;
     if (skipped) *skipped = amp->h_pinned->last_skipped;
@@ -798,15 +860,7 @@ try {
                              variance_buffers, weight16_buffers, num_weights, buffer_sizes, learning_rate,
                              beta1, beta2, epsilon, weight_decay, 0, true, l, lock))
         return rc;
-    // the event marks the arrival of this step's post-state in its ring slot
-    const uint64_t issue = amp->issued + 1;
-    const int slot = (int)(issue % kAmpMaxInFlight);
-    if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
-        // the step itself is enqueued; resynchronise the bookkeeping with the device
-        (void)amp_download(amp);
-        return -6;
-    }
-    amp->issued = issue;
+    amp->issued += 1;       // its post-state will arrive in the ring slot of this issue number, stamp last
     return 0;
 } catch (...) {
     note_exception();
@@ -858,7 +912,7 @@ try {
     if (int rc = amp_enqueue_fused(device, amp, a, b, gradient16_buffers, weight16_buffers, num_weights, buffer_sizes,
                                    learning_rate, beta1, beta2, epsilon, weight_decay, step_count, false, l, lock))
         return rc;
-    if (!hip_ok(hipStreamSynchronize(l.ctx->stream), "hipStreamSynchronize")) return -6;
+    if (!amp_wait_outcome(amp, amp->last_stamp, false)) return -6;
     amp->confirmed_issue = amp->issued;
     amp->confirmed_applied = amp->h_pinned->applied_steps;
     if (skipped) *skipped = amp->h_pinned->last_skipped;
@@ -888,13 +942,7 @@ try {
     if (int rc = amp_enqueue_fused(device, amp, a, b, gradient16_buffers, weight16_buffers, num_weights, buffer_sizes,
                                    learning_rate, beta1, beta2, epsilon, weight_decay, 0, true, l, lock))
         return rc;
-    const uint64_t issue = amp->issued + 1;
-    const int slot = (int)(issue % kAmpMaxInFlight);
-    if (!hip_ok(hipEventRecord(amp->ring_event[slot], l.ctx->stream), "hipEventRecord")) {
-        (void)amp_download(amp);
-        return -6;
-    }
-    amp->issued = issue;
+    amp->issued += 1;
     return 0;
 } catch (...) {
     note_exception();

@@ -282,7 +282,10 @@ int gm_amp_state_set_step_count(uintptr_t amp_state, int applied_steps);
  * Otherwise g = float(g16) * (1.0f / scale), the Adam rule of
  * execute_adam_step_mpsgraph, w16 = half(w'), counter++, and scale *= growth
  * when the counter reaches growth_interval; *skipped = 0.
- * The call synchronises the stream (it reports *skipped).  scale_out /
+ * The call returns once the step's outcome is known (it reports *skipped): the check has
+ * finished and the update, if any, is launched; like the fp32 steps the update itself completes
+ * on the library's stream, ahead of whatever is enqueued there next, and every call that hands
+ * data to the host waits for it (gm_synchronize waits explicitly).  scale_out /
  * growth_tracker_out (may be NULL) receive the state after the step.
  * -1 device 0; -3 no GPU; -4 a required handle is 0; -6 HIP error; -16 amp_state 0. */
 int execute_adam_amp_step(uintptr_t device, uintptr_t *weight_buffers,
