@@ -200,16 +200,23 @@ amp_adam_update_kernel(const Chunk *__restrict__ chunks, uint32_t slice_shift, S
     const uintx4 head = *reinterpret_cast<const uintx4 *>(pre);
     const unsigned long long seen = *overflow;
     const Chunk ch = chunks[blockIdx.x >> slice_shift];
+    __builtin_amdgcn_sched_barrier(0);     // all three fetches are issued before the first of them is waited for
     const uint32_t first_lane_element = (blockIdx.x & ((1u << slice_shift) - 1u)) * BLOCK * VEC;
     const bool found = seen == stamp;
-    if (post != nullptr && blockIdx.x == 0 && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 0, stamp);
+    // (the epilogue sits behind the update's loads and stores, not in front of them: a workgroup lives for a
+    // microsecond or two, and whatever stands between its start and its first global load shows in the bandwidth)
+    const bool epilogue = post != nullptr && blockIdx.x == 0;
     // (the weight pointer is never null; testing it here makes the compiler fetch the whole
     // descriptor before the branch instead of the count first and the addresses after it)
-    if (found | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr))
-        return;                                                        // step dropped, or an idle slice
+    if (found | (first_lane_element >= ch.count) | (ch.p[kSlotWeight] == nullptr)) {
+        // step dropped, or an idle slice
+        if (epilogue && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 0, stamp);
+        return;
+    }
     const float inv_scale = __uint_as_float(head.y);
     amp_pick_bias(prm, bias, (int)head.w);
     update_slice<AdamRule, VEC, NT, true, BLOCK>(ch, slice_shift, prm, inv_scale);
+    if (epilogue && threadIdx.x == 0) amp_advance(pre, post, host_mirror, found, 0, stamp);
 }
 
 // One lane's share in two halves, so that the kernel can issue its global loads, do its scalar
@@ -289,8 +296,11 @@ amp_adam_fused_kernel(const AmpDeviceState *__restrict__ pre, const Chunk *__res
     // (an empty bias table cannot occur either; testing it here brings its size and base in together
     // with the descriptors, so the pick below is a dozen scalar instructions and not another
     // fetch-and-wait in front of the global loads)
+    // (the dropped-step count is never negative either; testing it keeps all four words of the head alive up to
+    // this point: with a dead word among them the compiler reuses its register for the chunk's element count while
+    // the head is still in flight, and has to wait for the first descriptor before it may fetch the second)
     if ((slice * BLOCK * VEC >= a.count) | (a.p[kSlotWeight] == nullptr) | (b.p[kSlotWeight] == nullptr) | (head.y == 0u) |
-        (bias.count < 1) | (bias.base < 0))
+        (bias.count < 1) | (bias.base < 0) | ((int)head.z < 0))
         return;
     const bool b_is_current = head.x != 0u;
     const Chunk &in = b_is_current ? b : a;
