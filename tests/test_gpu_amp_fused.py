@@ -319,3 +319,89 @@ def test_in_place_and_one_pass_steps_share_one_loss_scale_state(dev):
             pair.compare(f"step {k} ({form})")
     finally:
         pair.close()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_mix_of_forms_waits_and_state_edits(dev, seed):
+    """One loss-scale state driven by a random program: bursts of one to six steps, each burst in place or in one
+    pass, waited for step by step or run ahead, with injected overflows, and between bursts now and then a restored
+    scale / clean-step counter or a step count set by the host.  The device keeps its state in two records that
+    swap roles with every step and tells finished steps by stamps in pinned memory: after every burst the counters,
+    the current set and every buffer must be the oracle's."""
+    lib, D = dev.lib, dev.handle
+    rng = np.random.default_rng(0xA11CE + seed)
+    sizes = [int(x) for x in rng.choice([1, 63, 256, 1000, 4097, 70001, 150_000], size=int(rng.integers(2, 6)))]
+    interval = int(rng.integers(2, 6))
+    pair = FusedPair(dev, [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes], HYPER, (4096.0, 2.0, 0.5, interval))
+    g_dev = [[dev.alloc(2 * n) for n in sizes] for _ in range(6)]
+    g_arr = [pkg.handle_array(hs) for hs in g_dev]
+    h = pair.h
+    skipped_total = 0
+    try:
+        for burst in range(30):
+            one_pass = bool(rng.integers(0, 2))
+            waited = bool(rng.integers(0, 2))
+            length = int(rng.integers(1, 7))
+            in_set = pair.current                        # an in-place burst works on the set current at its start
+            expected = []
+            for j in range(length):
+                g16 = scaled_g16(rng, sizes, np.float32(pair.st.scale))
+                if rng.random() < 0.25:
+                    t = int(rng.integers(0, len(sizes)))
+                    g16[t][int(rng.integers(0, sizes[t]))] = [0x7C00, 0xFC00, 0x7E00][(burst + j) % 3]
+                for hd, g in zip(g_dev[j], g16):
+                    dev.upload(hd, g)
+                count_before = int(pair.st.step_count)
+                sk = oracle().adam_amp(pair.w, g16, pair.m, pair.v, pair.w16, state=pair.st, **h)
+                skipped_total += sk
+                if one_pass and not sk:
+                    pair.current ^= 1
+                expected.append((sk, float(np.float32(pair.st.scale)), pair.st.growth_tracker, pair.current, count_before + 1))
+            a, b, cur = pair.c[0], pair.c[1], pair.c[in_set]
+            for j in range(length):
+                skipped, scale, tracker, now = ctypes.c_int(-1), ctypes.c_float(0), ctypes.c_int(-1), ctypes.c_int(-1)
+                if one_pass and waited:
+                    rc = lib.execute_adam_amp_step_fused(D, a["w"], a["m"], a["v"], b["w"], b["m"], b["v"], g_arr[j],
+                                                         pair.c_w16, pair.n, pair.bs, h["lr"], h["beta1"], h["beta2"],
+                                                         h["eps"], h["weight_decay"], expected[j][4], pair.amp,
+                                                         ctypes.byref(skipped), ctypes.byref(scale), ctypes.byref(tracker),
+                                                         ctypes.byref(now))
+                    assert (skipped.value, scale.value, tracker.value, now.value) == expected[j][:4], (burst, j)
+                elif one_pass:
+                    rc = lib.execute_adam_amp_step_fused_async(D, a["w"], a["m"], a["v"], b["w"], b["m"], b["v"], g_arr[j],
+                                                               pair.c_w16, pair.n, pair.bs, h["lr"], h["beta1"],
+                                                               h["beta2"], h["eps"], h["weight_decay"], pair.amp)
+                elif waited:
+                    rc = lib.execute_adam_amp_step(D, cur["w"], g_arr[j], cur["m"], cur["v"], pair.c_w16, pair.n, pair.bs,
+                                                   h["lr"], h["beta1"], h["beta2"], h["eps"], h["weight_decay"],
+                                                   expected[j][4], pair.amp, ctypes.byref(skipped), ctypes.byref(scale),
+                                                   ctypes.byref(tracker))
+                    assert (skipped.value, scale.value, tracker.value) == expected[j][:3], (burst, j)
+                else:
+                    rc = lib.execute_adam_amp_step_async(D, cur["w"], g_arr[j], cur["m"], cur["v"], pair.c_w16, pair.n,
+                                                         pair.bs, h["lr"], h["beta1"], h["beta2"], h["eps"],
+                                                         h["weight_decay"], pair.amp)
+                assert rc == 0, (rc, lib.gm_last_error(), burst, j)
+            scale, tracker, applied, skipped = ctypes.c_float(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+            assert lib.gm_amp_state_query(pair.amp, ctypes.byref(scale), ctypes.byref(tracker), ctypes.byref(applied),
+                                          ctypes.byref(skipped)) == 0
+            assert (scale.value, tracker.value, applied.value, skipped.value) == \
+                (float(np.float32(pair.st.scale)), pair.st.growth_tracker, pair.st.step_count, skipped_total), (burst, one_pass, waited)
+            assert lib.gm_amp_state_current_set(pair.amp) == pair.current
+            pair.compare(f"seed {seed} burst {burst}")
+            edit = rng.random()
+            if edit < 0.15:                               # a checkpoint's scale and counter are restored
+                new_scale = float(2.0 ** int(rng.integers(8, 15)))
+                new_tracker = int(rng.integers(0, interval))
+                assert lib.gm_amp_state_set(pair.amp, new_scale, new_tracker) == 0
+                pair.st.scale, pair.st.growth_tracker = new_scale, new_tracker
+            elif edit < 0.3:                              # the optimizer's step count is set by the host
+                new_count = int(rng.integers(0, 3000))
+                assert lib.gm_amp_state_set_step_count(pair.amp, new_count) == 0
+                pair.st.step_count = new_count
+        assert skipped_total > 5
+    finally:
+        pair.close()
+        for hs in g_dev:
+            for hd in hs:
+                dev.free(hd)
