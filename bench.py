@@ -51,16 +51,19 @@ BYTES_PER_PARAM = {"sgd": 20, "adam": 28, "rmsprop": 20, "adagrad": 20, "adadelt
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # file (summary and commands: profiles/adam_c5_1b_hbm_traffic.md); None where not measured.
 MEASURED_HBM_TRAFFIC = {("c5", "adam"): 2.8359e10,
-                        # the three launches of one mixed-precision step: check 2.026e9 + update 2.8345e10
+                        # the launches of one in-place mixed-precision step: check 2.026e9 + update 2.8345e10
                         ("c5", "adam_amp"): 3.0385e10,
                         # the one-pass step over ping-pong state: a single update launch
                         ("c5", "adam_amp_one_pass"): 2.8375e10,
+                        # configs 3 and 4 (profiles/c3_c4_hbm_traffic.md)
+                        ("c3-rmsprop", "rmsprop"): 5.0643e8, ("c3-adagrad", "adagrad"): 5.0644e8,
+                        ("c3-adadelta", "adadelta"): 7.0642e8, ("c3-nadam", "nadam"): 7.0640e8,
+                        ("c4", "adam"): 3.5019e9, ("c4", "adam_amp"): 3.7522e9, ("c4", "adam_amp_one_pass"): 3.5039e9,
                         # bytes per step, summed over the passes of a 10-pair step (profiles/lbfgs_c5_1b_hbm_traffic.md)
                         ("lbfgs-c5", 10): 352.68 * 1012301824}
-TRAFFIC_SOURCE = {("c5", "adam"): "profiles/adam_c5_1b_hbm_traffic.md",
-                  ("c5", "adam_amp"): "profiles/adam_c5_1b_hbm_traffic.md",
-                  ("c5", "adam_amp_one_pass"): "profiles/adam_c5_1b_hbm_traffic.md",
-                  ("lbfgs-c5", 10): "profiles/lbfgs_c5_1b_hbm_traffic.md"}
+TRAFFIC_SOURCE = {("lbfgs-c5", 10): "profiles/lbfgs_c5_1b_hbm_traffic.md"}
+TRAFFIC_SOURCE.update({k: "profiles/adam_c5_1b_hbm_traffic.md" for k in MEASURED_HBM_TRAFFIC if k[0] == "c5"})
+TRAFFIC_SOURCE.update({k: "profiles/c3_c4_hbm_traffic.md" for k in MEASURED_HBM_TRAFFIC if k[0][:2] in ("c3", "c4")})
 
 
 def traffic_fields(key):
