@@ -285,6 +285,40 @@ def test_amp_over_many_tiny_tensors(dev):
         pair.close()
 
 
+def test_a_list_without_elements_still_advances_the_loss_scale_state(dev):
+    """Every tensor empty: there is no check or update launch to carry the epilogue, yet each step counts as
+    applied (no gradient overflowed), the clean-step counter runs and the scale grows at the interval, with and
+    without the host waiting for the step."""
+    lib, pkg = dev.lib, load_package()
+    bufs = {k: [dev.alloc(16, zero=True) for _ in range(2)] for k in ("w", "g16", "m", "v", "w16")}
+    c = {k: pkg.handle_array(v) for k, v in bufs.items()}
+    bs = pkg.int_array([0, 0])
+    amp = lib.gm_amp_state_create(dev.handle, 1024.0, 2.0, 0.5, 3)
+    st = oracle().amp_state(1024.0, 2.0, 0.5, 3)
+    none = [np.zeros(0, np.float32)] * 2
+    none16 = [np.zeros(0, np.uint16)] * 2
+    try:
+        for t in range(4):
+            got = amp_step_gpu(dev, pkg, c, bs, 2, HYPER, t + 1, amp)
+            want = oracle().adam_amp(none, none16, none, none, none16, state=st, **HYPER)
+            assert got == (want, float(np.float32(st.scale)), st.growth_tracker) and want == 0
+        assert (float(np.float32(st.scale)), st.growth_tracker, st.step_count) == (2048.0, 1, 4)
+        for t in range(3):
+            rc = lib.execute_adam_amp_step_async(dev.handle, c["w"], c["g16"], c["m"], c["v"], c["w16"], 2, bs,
+                                                 HYPER["lr"], HYPER["beta1"], HYPER["beta2"], HYPER["eps"],
+                                                 HYPER["weight_decay"], amp)
+            assert rc == 0, (rc, lib.gm_last_error())
+        scale, tracker, applied, skipped = ctypes.c_float(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        assert lib.gm_amp_state_query(amp, ctypes.byref(scale), ctypes.byref(tracker), ctypes.byref(applied),
+                                      ctypes.byref(skipped)) == 0
+        assert (scale.value, tracker.value, applied.value, skipped.value) == (4096.0, 1, 7, 0)
+    finally:
+        lib.gm_amp_state_destroy(amp)
+        for hs in bufs.values():
+            for h in hs:
+                dev.free(h)
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_random_lists_scales_and_injections(dev, seed):
     """Tensor lists, initial scales, growth intervals, hyper-parameters and non-finite injections (+inf, -inf, two
