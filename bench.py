@@ -178,6 +178,7 @@ def cpu_baseline_amp(sizes, hyper, grad_std, budget_params=96_000_000, target_se
         step()
     dt = time.perf_counter() - t0
     return {"value": total * steps / dt, "unit": "params/s", "cores": threads, "kind": "port",
+            "sample_params": total, "sample_steps": steps, "sample_seconds": dt,
             "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} mixed-precision steps in "
                       f"{dt:.1f} s, oracle/oracle.c (eight-lane AVX2 + F16C form where the host has them) with OpenMP "
                       f"on {threads} threads of {os.cpu_count()} ({cpu_model()})"}
@@ -210,6 +211,7 @@ def cpu_baseline(sizes, rule, hyper, grad_std, budget_params=96_000_000, target_
         run.step(g)
     dt = time.perf_counter() - t0
     return {"value": total * steps / dt, "unit": "params/s", "cores": threads, "kind": "port",
+            "sample_params": total, "sample_steps": steps, "sample_seconds": dt,
             "sample": f"first {len(chosen)} tensors ({total} params) of the workload, {steps} steps in "
                       f"{dt:.1f} s, oracle/oracle.c with OpenMP on {threads} threads of {os.cpu_count()} "
                       f"({cpu_model()})"}
@@ -516,7 +518,8 @@ def compact_line(results, records_file):
     cpu = h.get("cpu_baseline")
     line["cpu_baseline"] = None if cpu is None else {
         "value": _sig(cpu["value"]), "unit": cpu["unit"], "cores": cpu["cores"], "kind": cpu["kind"],
-        "sample": cpu["sample"][:64]}
+        "sample": (f"{cpu['sample_params']} params x {cpu['sample_steps']} steps, {cpu['sample_seconds']:.1f} s, oracle.c OpenMP"
+                   if "sample_params" in cpu else cpu["sample"][:64])}
     amp = h.get("amp")
     if amp:
         form = lambda r: {"frac": _sig(r["roofline"]["frac"], 4), "ms_per_step": _sig(r["ms_per_step"], 4)}

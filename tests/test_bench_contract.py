@@ -78,7 +78,8 @@ def synthetic_records():
                       "kernel_ms": 4.302727222442627, "kernel_ms_median": 4.3, "kernel_ms_min": 4.29,
                       "copy_kernel_gbs": 6617.441724517294, "frac_of_copy_kernel": 0.9872677298195458, "note": prose,
                       "frac_hbm": 0.7912345678, "achieved_hbm": 6329.87654321, "footprint_bytes": 400000000}
-    cpu = {"value": 5644320252.590273, "unit": "params/s", "cores": 16, "kind": "port", "sample": prose}
+    cpu = {"value": 5644320252.590273, "unit": "params/s", "cores": 16, "kind": "port", "sample": prose,
+           "sample_params": 95543296, "sample_steps": 740, "sample_seconds": 12.04567}
     form = lambda k: {"value": 213929119892.47342, "unit": "params/s", "ms_per_step": 4.731949650000011, "dtype": prose[:60],
                       "skipped_steps": 0, "roofline": roof(k), "form": prose,
                       "async": {"value": 2.1e11, "ms_per_step": 4.718167249999983, "kernel_ms": 4.712443923950195,
