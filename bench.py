@@ -9,14 +9,16 @@ parameters in 400 tensors shaped like transformer blocks.
 Prints ONE JSON line: params updated per second (whole job), ms per step, the roofline of
 the dominant kernel (algorithmic bytes per launch / launch duration measured with HIP
 events on the library's own stream, against MI355X's 8 TB/s HBM peak), the same figures for
-the mixed-precision (fp16 gradient) Adam step ("amp": the one-pass form over ping-pong state
-leads, "amp.in_place" is the form that keeps one set of state and reads the gradients twice; each
-also without the per-step host wait under "async"), and the CPU oracle timed on this host's cores
-on a bounded sample of the same workload.
+the mixed-precision (fp16 gradient) Adam step ("amp": the form that updates in place, which
+StepAMP runs by default, and the one-pass form over ping-pong state; each also without the
+per-step host wait under "async"), and the CPU oracle timed on this host's cores on a bounded
+sample of the same workload.
 
-Without --workload, every benchmark configuration runs, each in a process of its own: the line
-is the headline configuration's, and "configs" holds the same record for configurations 1 to 4
-(--workload all adds the L-BFGS workloads and the buffer primitives; --workload NAME runs one).
+Without --workload, every benchmark configuration runs, each in a process of its own.  The one
+line printed is then a short one (under 2 KB): the headline configuration's record, and under
+"configs" the figures of configurations 1 to 4; the full records go to a file the line names
+(--workload all adds the L-BFGS workloads and the buffer primitives; --workload NAME runs one
+workload in this process and prints its full record).
 """
 import argparse
 import ctypes
@@ -33,6 +35,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "go-metal_amd"))      # workloads.py: the configurations' tensor lists
 
 HBM_PEAK_GBS = 8000.0
+RECORDS_FILE = os.path.join("gpurun_out", "bench_configs.json")     # full per-configuration records of the default run
 LINE_LIMIT = 1960         # bytes of the default run's final line: the driver keeps the tail of stdout
 ROTATE_C3 = 6            # copies of the 25M list stepped in turn by the default run: 6 x 300-400 MB
 STATE_PHASES = (512 << 10, 1536 << 10, 1 << 20)     # host/memory_manager.hpp, kStatePhases
@@ -562,7 +565,7 @@ def compact_line(results, records_file):
 
 def run_children(args, names):
     """Each named workload as a child process, started before this process has made any GPU call (it never
-    makes one).  The full records go to gpurun_out/bench_configs.json; the last line printed is the headline
+    makes one).  The full records go to the file RECORDS_FILE names; the last line printed is the headline
     configuration's, with the other configurations' figures under "configs" (compact_line)."""
     import subprocess
     results = {}
@@ -584,12 +587,10 @@ def run_children(args, names):
         print(f"running {name}", file=sys.stderr, flush=True)
         out = subprocess.run(cmd, check=True, stdout=subprocess.PIPE, text=True).stdout
         results[name] = json.loads(out.strip().splitlines()[-1])
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    os.makedirs(out_dir, exist_ok=True)
-    records_file = os.path.join("gpurun_out", "bench_configs.json")
-    with open(os.path.join(ROOT, records_file), "w") as f:
+    os.makedirs(os.path.dirname(os.path.join(ROOT, RECORDS_FILE)), exist_ok=True)
+    with open(os.path.join(ROOT, RECORDS_FILE), "w") as f:
         json.dump(results, f, indent=1)
-    print(compact_line(results, records_file), flush=True)
+    print(compact_line(results, RECORDS_FILE), flush=True)
 
 
 def main():

@@ -177,7 +177,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
 @pytest.mark.gpu
 def test_default_run_ends_with_one_short_line_the_driver_can_parse():
     """The command the driver runs (no workload named), shortened: every configuration in a process of its own,
-    the full records in gpurun_out/bench_configs.json, and stdout = ONE line under 2 KB."""
+    the full records in the file the line names, and stdout = ONE line under 2 KB."""
     r = subprocess.run([sys.executable, BENCH, "--gpus", "1", "--steps", "2", "--warmup", "1", "--cpu-seconds", "0.3"],
                        capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stderr[-2000:]
