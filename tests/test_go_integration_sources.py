@@ -29,15 +29,35 @@ def split_top_level(args):
     return parts
 
 
-def header_prototypes():
+def header_prototypes(with_types=False):
     text = open(os.path.join(ROOT, "include", "gometal_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = re.sub(r"//[^\n]*", "", text)
     protos = {}
     for m in re.finditer(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(([^()]*)\)\s*;", text):
         name, args = m.group(1), m.group(2).strip()
-        protos[name] = 0 if args in ("", "void") else len(split_top_level(args))
+        params = [] if args in ("", "void") else split_top_level(args)
+        protos[name] = [c_kind(p) for p in params] if with_types else len(params)
     return protos
+
+
+def c_kind(param):
+    """pointer / float / int / uintptr_t of a C parameter declaration."""
+    if "*" in param:
+        return "pointer"
+    for kind in ("float", "uintptr_t", "int"):
+        if re.search(rf"\b{kind}\b", param):
+            return kind
+    return param
+
+
+def go_kind(arg):
+    """The same classification of an argument expression of a cgo call."""
+    arg = arg.strip()
+    if arg.startswith("&") or arg.startswith("first("):
+        return "pointer"
+    m = re.match(r"C\.([A-Za-z_0-9]+)\(", arg)
+    return m.group(1) if m else arg
 
 
 def go_c_calls(path):
@@ -54,7 +74,8 @@ def go_c_calls(path):
         while depth:
             depth += {"(": 1, ")": -1}.get(text[i], 0)
             i += 1
-        calls.append((name, len(split_top_level(text[m.end():i - 1])), text.count("\n", 0, m.start()) + 1))
+        args = split_top_level(text[m.end():i - 1])
+        calls.append((name, len(args), text.count("\n", 0, m.start()) + 1, args))
     return calls
 
 
@@ -70,7 +91,7 @@ def test_every_c_function_the_go_wrappers_call_is_declared_with_that_arity():
     assert protos["gm_allocate_buffer_phased"] == 4 and protos["gm_amp_state_query"] == 5
     seen = set()
     for path in go_files():
-        for name, nargs, line in go_c_calls(path):
+        for name, nargs, line, _ in go_c_calls(path):
             where = f"{os.path.relpath(path, ROOT)}:{line}"
             assert name in protos, f"{where}: C.{name} is not declared in include/gometal_hip.h"
             assert nargs == protos[name], f"{where}: C.{name} called with {nargs} arguments, declared with {protos[name]}"
@@ -79,6 +100,19 @@ def test_every_c_function_the_go_wrappers_call_is_declared_with_that_arity():
             "execute_adam_amp_step_fused_async", "gm_allocate_buffer_phased", "gm_amp_state_create",
             "gm_amp_state_destroy", "gm_amp_state_query", "gm_amp_state_set", "gm_amp_state_set_step_count",
             "gm_amp_state_current_set", "gm_amp_state_set_current_set", "gm_synchronize"} <= seen
+
+
+def test_every_argument_of_a_cgo_call_has_the_kind_the_header_declares():
+    """Position by position: a pointer where the header has a pointer, C.float where it has float, C.int where it has
+    int, C.uintptr_t where it has uintptr_t (two arguments swapped in a call would compile in C and fail here)."""
+    protos = header_prototypes(with_types=True)
+    checked = 0
+    for path in go_files():
+        for name, _, line, args in go_c_calls(path):
+            got = [go_kind(a) for a in args]
+            assert got == protos[name], f"{os.path.relpath(path, ROOT)}:{line}: C.{name}({got}) against {protos[name]}"
+            checked += len(args)
+    assert checked > 90
 
 
 def test_go_files_are_plausible_go():
