@@ -152,12 +152,15 @@ public:
     void Cleanup() override;
 
     // ---- mixed precision (additive; constants from training/model_trainer.go:258-270) ----
-    // Creates the device-resident loss-scale state.  Call once before StepAMP.
+    // Creates the device-resident loss-scale state.  Call before StepAMP.  A further call replaces the state
+    // (steps in flight finish first; with ping-pong state on, the new state is told which set is current).
     Error EnableMixedPrecision(float initialScale = 65536.0f, float growthFactor = 2.0f,
                                float backoffFactor = 0.5f, int growthInterval = 2000);
     // One step on fp16 gradients of the scaled loss.  Returns skipped = true (and leaves
     // StepCount, weights and moments untouched) when a gradient holds inf / NaN.
-    // weight16Buffers may be empty (no fp16 weight copy).
+    // weight16Buffers may be empty (no fp16 weight copy).  Updates in place unless EnablePingPong
+    // was called: the caller's own fp32 weight buffers hold the current weights after every step.
+    // Returns when the outcome is known; the update completes on the library's stream like an fp32 Step.
     std::pair<bool, Error> StepAMP(const std::vector<Pointer> &gradient16Buffers,
                                    const std::vector<Pointer> &weight16Buffers);
     // The same step without waiting for it: no result is returned, and up to 7 steps run ahead
