@@ -62,6 +62,19 @@ func Synchronize(device unsafe.Pointer) error {
 	return nil
 }
 
+// BiasCorrections returns 1 - beta1^step and 1 - beta2^step exactly as the Adam and NAdam entry points compute
+// them (the C library's powf in float32, bridge_optimizer.m:398-399).
+func BiasCorrections(beta1, beta2 float32, step int) (bc1, bc2 float32) {
+	var a, b C.float
+	C.gm_bias_corrections(C.float(beta1), C.float(beta2), C.int(step), &a, &b)
+	return float32(a), float32(b)
+}
+
+// NadamMuNext returns NAdam's momentum schedule at step + 1 as the entry point computes it (bridge_optimizer.m:2066).
+func NadamMuNext(beta1 float32, step int) float32 {
+	return float32(C.gm_nadam_mu_next(C.float(beta1), C.int(step)))
+}
+
 // CreateAMPState creates the device-resident loss-scale state of the mixed-precision step
 // (defaults of training/model_trainer.go:258-270: 65536, 2, 0.5, 2000).
 func CreateAMPState(device unsafe.Pointer, initialScale, growthFactor, backoffFactor float32, growthInterval int) (unsafe.Pointer, error) {

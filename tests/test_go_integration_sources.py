@@ -162,3 +162,23 @@ def test_hooks_named_in_the_go_files_exist():
     assert "kStatePhases[3] = {512 << 10, 1536 << 10, 1 << 20}" in hpp and "[3]int{512 << 10, 1536 << 10, 1 << 20}" in mem
     assert "kShadowWeightPhase = 1 << 20" in hpp and "ShadowWeightPhase = 1 << 20" in mem
     assert "kPhasedMinBytes = 16 << 20" in hpp and "PhasedMinBytes = 16 << 20" in mem
+
+
+def test_go_oracle_restates_every_statement_the_c_oracle_cites():
+    """oracle_cpu.go is the Go form of oracle/oracle.c's update rules (it cannot be run here).  Both annotate every
+    statement with the line of bridge_optimizer.m it follows: each citation of the C rules must appear in the Go file,
+    the same number of times, so a statement dropped or doubled in the translation shows."""
+    c_text = open(os.path.join(ROOT, "oracle", "oracle.c")).read()
+    rules = c_text[c_text.index("void gm_oracle_sgd_step"):c_text.index("/* ---- fp16 casts")]
+    go_text = open(os.path.join(GO, "optimizer", "oracle_cpu.go")).read()
+    go_rules = go_text[go_text.index("func OracleSGDStep"):go_text.index("// Float16ToFloat32")]
+    cite = lambda text, pattern: sorted(re.findall(pattern, text))
+    c_cites = cite(rules, r"/\* :(\d+(?:-\d+)?) \*/")
+    go_cites = sorted(a or b for a, b in re.findall(r"// :(\d+(?:-\d+)?)[ \t]*\n|// :(\d+(?:-\d+)?)$", go_rules, flags=re.M))
+    assert len(c_cites) > 80
+    assert go_cites == c_cites, (sorted(set(c_cites) - set(go_cites)), sorted(set(go_cites) - set(c_cites)))
+    # and the same operators in the same order, statement by statement, for the Adam element
+    c_adam = c_text[c_text.index("static inline void adam_element"):c_text.index("/* bridge_optimizer.m:360-641 */")]
+    go_adam = go_text[go_text.index("func adamElement"):go_text.index("// OracleAdamStep")]
+    ops = lambda text, marker: re.findall(r"= [^;\n]*?([*/+-])[^;\n]*?" + marker, text)
+    assert ops(c_adam, r";\s*/\* :") == ops(go_adam, r"\)\s*// :") and len(ops(c_adam, r";\s*/\* :")) >= 12
