@@ -85,19 +85,27 @@ struct AmpBiasTable {
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
 amp_overflow_check_kernel(const Chunk *__restrict__ chunks, unsigned long long *__restrict__ overflow, int reverse,
-                          unsigned long long stamp)
+                          unsigned long long stamp, uint32_t num_chunks, uint32_t split_shift)
 {
     __shared__ unsigned int wave_hit[kBlock / 64];
+    // A list of few chunks is checked by several workgroups per chunk (1 << split_shift of them, each taking
+    // a run of whole 2048-element rows), so that a 1M-parameter tensor in sixteen 65536-element chunks is not
+    // read by sixteen workgroups; lists of a thousand chunks and more take one workgroup per chunk.
+    const uint32_t c = blockIdx.x >> split_shift;
+    const uint32_t part = blockIdx.x & ((1u << split_shift) - 1u);
     // reverse: the table is walked from its end, so that the check finishes on the gradients the
     // update pass reads first (what is left of them in the memory-side cache is then the nearest)
-    const Chunk ch = chunks[reverse ? gridDim.x - 1u - blockIdx.x : blockIdx.x];
+    const Chunk ch = chunks[reverse ? num_chunks - 1u - c : c];
     const unsigned short *g = reinterpret_cast<const unsigned short *>(ch.p[kSlotGrad]);
+    const uint32_t per_part = (((ch.count + (1u << split_shift) - 1u) >> split_shift) + 2047u) & ~2047u;
+    const uint32_t lo = part * per_part < ch.count ? part * per_part : ch.count;
+    const uint32_t hi = ch.count - lo < per_part ? ch.count : lo + per_part;
     unsigned int bad = 0;
-    uint32_t done = 0;
+    uint32_t done = lo;
     if (ch.flags & kRecGrad16VectorOk) {
-        const uint32_t n8 = ch.count >> 3;
+        const uint32_t n8 = hi >> 3;
         const uintx4 *g8 = reinterpret_cast<const uintx4 *>(g);
-        for (uint32_t base = threadIdx.x; base < n8; base += kBlock * kCheckUnroll) {
+        for (uint32_t base = (lo >> 3) + threadIdx.x; base < n8; base += kBlock * kCheckUnroll) {
             uintx4 v[kCheckUnroll];
 #pragma unroll
             for (int u = 0; u < kCheckUnroll; u++) {
@@ -107,15 +115,15 @@ amp_overflow_check_kernel(const Chunk *__restrict__ chunks, unsigned long long *
 #pragma unroll
             for (int u = 0; u < kCheckUnroll; u++) {
 #pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    const unsigned int e = v[u][c] & 0x7C007C00u;
+                for (int c4 = 0; c4 < 4; c4++) {
+                    const unsigned int e = v[u][c4] & 0x7C007C00u;
                     bad |= ((e & 0xFFFFu) == 0x7C00u) | ((e >> 16) == 0x7C00u);
                 }
             }
         }
-        done = n8 << 3;
+        done = n8 << 3 > lo ? n8 << 3 : lo;
     }
-    for (uint32_t i = done + threadIdx.x; i < ch.count; i += kBlock)
+    for (uint32_t i = done + threadIdx.x; i < hi; i += kBlock)
         bad |= ((stream_load<false>(g + i) & 0x7C00u) == 0x7C00u);
 
     const unsigned long long ballot = __ballot(bad != 0);
@@ -733,12 +741,23 @@ static int amp_enqueue(uintptr_t device, AmpState *amp, uintptr_t *weight_buffer
     unsigned long long *overflow = &amp->d_block->overflow;
 
     if (chunks > 0) {
-        // the check walks the whole table, one workgroup per chunk of either segment
+        // the check walks the whole table: one workgroup per chunk of either segment, or several per chunk when
+        // the list has few chunks (rows of 2048 elements are not split)
         const int reverse = l.ctx->amp_check_reverse.load();
+        uint32_t split_shift = 0;
+        {
+            uint32_t smallest = 0;
+            for (int k = 0; k < l.plan->num_segments; k++)
+                if (l.plan->segment[k].num_chunks > 0 &&
+                    (smallest == 0 || (uint32_t)l.plan->segment[k].chunk_elements < smallest))
+                    smallest = (uint32_t)l.plan->segment[k].chunk_elements;
+            while ((chunks << split_shift) < 1024u && (smallest >> (split_shift + 1)) >= 2048u) split_shift++;
+        }
+        const uint32_t check_grid = chunks << split_shift;
         if (nt && l.ctx->amp_check_nontemporal.load())
-            amp_overflow_check_kernel<true><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, overflow, reverse, stamp);
+            amp_overflow_check_kernel<true><<<check_grid, kBlock, 0, st>>>(l.plan->d_chunks, overflow, reverse, stamp, chunks, split_shift);
         else
-            amp_overflow_check_kernel<false><<<chunks, kBlock, 0, st>>>(l.plan->d_chunks, overflow, reverse, stamp);
+            amp_overflow_check_kernel<false><<<check_grid, kBlock, 0, st>>>(l.plan->d_chunks, overflow, reverse, stamp, chunks, split_shift);
         // the first update launch of the step carries the epilogue, so that the host learns the outcome as soon as
         // the check has finished (a second segment's launch reads the same pre-state, which nothing writes)
 #define GM_LAUNCH_AMP(V, N, B) amp_adam_update_kernel<V, N, B><<<g.grid, B, 0, st>>>(g.chunks, g.shift, p, pre, overflow, bias, stamp, \

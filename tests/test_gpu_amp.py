@@ -285,6 +285,51 @@ def test_amp_over_many_tiny_tensors(dev):
         pair.close()
 
 
+@pytest.mark.parametrize("misalign", [0, 1])
+def test_overflow_anywhere_in_a_list_of_few_large_chunks_is_seen(dev, misalign):
+    """One tensor of a million elements is cut into sixteen 65536-element chunks, and the in-place step's check then
+    runs several workgroups per chunk, each over a run of 2048-element rows: an inf / NaN at the first and last
+    element of the tensor, of a chunk, of a row, in the ragged tail and at random places must each drop the step
+    (and a clean step in between must not).  misalign: the gradient view starts 2 bytes off, which takes the
+    element-by-element path."""
+    lib, pkg = dev.lib, load_package()
+    n = (1 << 20) + 77
+    rng = np.random.default_rng(91 + misalign)
+    w = rng.normal(0, 0.02, n).astype(np.float32)
+    bufs = {"w": dev.from_numpy(w), "m": dev.alloc(4 * n, zero=True), "v": dev.alloc(4 * n, zero=True),
+            "w16": dev.alloc(2 * n, zero=True)}
+    g_parent = dev.alloc(2 * n + 16)
+    g_view = g_parent + 2 * misalign
+    c = {k: pkg.handle_array([h]) for k, h in bufs.items()}
+    c["g16"] = pkg.handle_array([g_view])
+    bs = pkg.int_array([4 * n])
+    amp = lib.gm_amp_state_create(dev.handle, 1024.0, 2.0, 0.5, 1000)
+    clean = (rng.normal(0, 1e-3, n) * 1024.0).astype(np.float16).view(np.uint16)
+    places = [0, 1, 2047, 2048, 65535, 65536, 65536 + 2047, 15 * 65536, (1 << 20) - 1, 1 << 20, n - 9, n - 1]
+    places += [int(x) for x in rng.integers(0, n, 12)]
+    try:
+        applied = 0
+        for k, place in enumerate(places):
+            g = clean.copy()
+            g[place] = [0x7C00, 0xFC00, 0x7E01][k % 3]
+            padded = np.zeros(n + 8, np.uint16)
+            padded[misalign:misalign + n] = g
+            dev.upload(g_parent, padded)
+            got = amp_step_gpu(dev, pkg, c, bs, 1, HYPER, applied + 1, amp)
+            assert got[0] == 1, (place, got)
+            if k % 4 == 0:                               # a clean step between dropped ones
+                padded[misalign:misalign + n] = clean
+                dev.upload(g_parent, padded)
+                got = amp_step_gpu(dev, pkg, c, bs, 1, HYPER, applied + 1, amp)
+                assert got[0] == 0, (place, got)
+                applied += 1
+        assert np.array_equal(dev.to_numpy(bufs["w"], n) != w, np.ones(n, bool)) or applied > 0
+    finally:
+        lib.gm_amp_state_destroy(amp)
+        for h in list(bufs.values()) + [g_parent]:
+            dev.free(h)
+
+
 def test_a_list_without_elements_still_advances_the_loss_scale_state(dev):
     """Every tensor empty: there is no check or update launch to carry the epilogue, yet each step counts as
     applied (no gradient overflowed), the clean-step counter runs and the scale grows at the interval, with and
