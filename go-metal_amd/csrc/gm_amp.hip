@@ -537,8 +537,9 @@ try {
     s->ctx = ctx;
     bool ok = hip_ok(hipMalloc(&s->d_block, sizeof(AmpDeviceBlock)), "hipMalloc(amp state)") &&
               hip_ok(hipMemsetAsync(s->d_block, 0, sizeof(AmpDeviceBlock), ctx->stream), "hipMemsetAsync(amp state)") &&
+              // coherent whatever HIP_HOST_COHERENT says: the host reads stamps while the kernel that wrote them runs
               hip_ok(hipHostMalloc(&s->h_pinned, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState),
-                                   hipHostMallocDefault), "hipHostMalloc(amp state)");
+                                   hipHostMallocCoherent), "hipHostMalloc(amp state)");
     if (ok) {
         std::memset(s->h_pinned, 0, (kAmpMaxInFlight + 1) * sizeof(AmpDeviceState));
         s->h_pinned->scale = init_scale;
