@@ -287,3 +287,13 @@ def test_config5_mixed_precision_full_size_20_steps(dev):
     inject = {0: (7, 5, 0x7C00), 6: (len(sizes) - 3, 1234, 0xFC00), 13: (2, 4096 * 11008 - 1, 0x7E00)}
     trace = run_schedule(dev, "config 5 mixed precision", sizes, hyper, 20, inject, {0, 1, 9, 19}, seed=5)
     assert [t[0] for t in trace].count(1) == 3 and trace[-1][1] == 8192.0 and trace[-1][3] == 17
+
+
+def test_a_tensor_of_the_largest_size_the_abi_can_name(dev):
+    """2^29 - 1 elements (2^31 - 4 bytes of fp32, the largest C int in bytes that is a whole number of floats) next to
+    a three-element tensor and a 2^28-element one, both forms, three steps; the middle step is dropped for a NaN in
+    the large tensor's last element."""
+    sizes = [2 ** 29 - 1, 3, 2 ** 28]
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4)
+    trace = run_schedule(dev, "largest tensor", sizes, hyper, 3, {1: (0, sizes[0] - 1, 0x7E00)}, {0, 1, 2}, seed=6)
+    assert [t[0] for t in trace] == [0, 1, 0] and trace[-1][1] == 32768.0 and trace[-1][3] == 2

@@ -14,11 +14,11 @@ pytestmark = pytest.mark.gpu
 NTHREADS = min(16, os.cpu_count() or 1)
 
 
-def run_full_size(rule, hyper, steps, checkpoints):
+def run_full_size(rule, hyper, steps, checkpoints, sizes=None):
     dev = gpu_device()
     if dev is None:
         pytest.fail("libgometal_hip.so is missing or no GPU is usable: GPU tests cannot run")
-    sizes = transformer_block_sizes()
+    sizes = transformer_block_sizes() if sizes is None else sizes
     # weights and two gradient sets are generated on the device and read back for the oracle
     lib, D = dev.lib, dev.handle
     gpu = GpuRun(dev, rule, hyper, [np.empty(0, np.float32)] * 0)   # placeholder object, filled below
@@ -73,6 +73,16 @@ def test_every_other_rule_over_the_1b_list(rule, hyper):
     on, the widest variant of each rule (Nesterov; RMSProp with momentum and centering: nine streams): three
     steps, compared after the last one."""
     run_full_size(rule, hyper, 3, (3,))
+
+
+def test_tensors_of_the_largest_size_the_abi_can_name():
+    """`sizes` are C ints in bytes, so the longest tensor a call can name has 2^29 - 1 elements (2^31 - 4 bytes, which
+    the allocator rounds up to 2^31).  Two of them with a five-element tensor in between: every byte offset above
+    2^31 inside the second large buffer, its last (odd) element and the tiny tensor's neighbours are the oracle's
+    after two steps of Adam with weight decay."""
+    top = 2 ** 29 - 1
+    run_full_size("adam", dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-4), 2, (2,),
+                  sizes=[top, 5, top])
 
 
 def test_adam_over_the_1b_list_through_the_optimizer_object():

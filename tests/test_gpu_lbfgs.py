@@ -345,8 +345,9 @@ def test_c5_size_dot_and_plain_step(dev):
 
 
 def test_dot_with_three_tree_levels(dev):
-    # more than 1024 * 1024 slices (1.2e9 elements): a plain level, then the fused last two
-    sizes = [450_000_000, 450_000_000, 300_000_000]
+    # more than 1024 * 1024 slices (1.29e9 elements): a plain level, then the fused last two; the first tensor has
+    # the largest size a C int in bytes can name (2^31 - 4), with a ragged last slice
+    sizes = [2 ** 29 - 1, 450_000_000, 300_000_000]
     lib, D = dev.lib, dev.handle
     ha = [dev.alloc(4 * k) for k in sizes]
     hb = [dev.alloc(4 * k) for k in sizes]
@@ -355,7 +356,7 @@ def test_dot_with_three_tree_levels(dev):
             assert lib.gm_fill_normal_f32(D, ha[i], k, 900 + i, 0.0, 1.0) == 0
             assert lib.gm_fill_normal_f32(D, hb[i], k, 950 + i, 0.5, 1.0) == 0
         out = ctypes.c_float()
-        print("dot product over 1.2e9 elements", flush=True)
+        print("dot product over 1.29e9 elements", flush=True)
         assert lib.gm_lbfgs_dot(D, pkg.handle_array(ha), pkg.handle_array(hb), 3, pkg.int_array([4 * k for k in sizes]),
                                 ctypes.byref(out)) == 0
         a = [dev.to_numpy(h, k) for h, k in zip(ha, sizes)]
